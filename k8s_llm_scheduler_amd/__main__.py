@@ -375,6 +375,11 @@ def cmd_e2e(args, cfg: Config) -> int:
 
 
 def main(argv: Optional[list] = None) -> int:
+    argv = sys.argv[1:] if argv is None else list(argv)
+    if argv and argv[0] in ("replay", "generate"):   # token-id front ends of the engine (engine/replay_cli.py)
+        from .engine import replay_cli
+
+        return {"replay": replay_cli.cmd_replay, "generate": replay_cli.cmd_generate}[argv[0]](argv[1:])
     ap = argparse.ArgumentParser(prog="k8s_llm_scheduler_amd", description=__doc__.splitlines()[0])
     ap.add_argument("command", nargs="?", default="run", choices=["run", "verify", "smoke", "e2e"])
     ap.add_argument("--config", default=None, help="config.yaml (default: $SCHEDULER_CONFIG or ./config.yaml)")

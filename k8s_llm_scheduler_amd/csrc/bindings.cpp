@@ -110,6 +110,32 @@ int k8s_pgemm4_config(int cfg, int* bp, int* bq, int* lds_bytes);
 int k8s_pgemm4_plan(int M, int N_out, int K, int epi, int cfg, int splits, int* nwg, long long* slab_elems);
 int k8s_pgemm4(void* out, float* slab, const void* x, const void* W, int M, int N_out, int K, int epi, int cfg,
                int splits, int group_m, const void* res, int rms, float eps, hipStream_t s);
+int k8s_embed_rows(float* out, const int* ids, const void* table, int T, int W, int vocab, int f32, hipStream_t s);
+int k8s_resnorm(float* x, const void* branch, float mult, const void* rowvec, const void* w, float offset, float eps,
+                void* out, int T, int W, int f32, hipStream_t s);
+int k8s_act(void* out, const void* x, int T, int F, int kind, float limit, float alpha, int f32, hipStream_t s);
+int k8s_gemm_any(void* C, const void* A, const void* W, int M, int N, int K, long lda, long ldw, long ldc, int batch,
+                 long sA, long sW, long sC, const int* a_rows, const int* tiles, int ntiles, int in_f32, int out_f32,
+                 hipStream_t s);
+int k8s_token_shift(void* out, const void* h, const void* mu, const void* state, const int* cu_q, const int* tok_seq,
+                    const int* seq_slots, const int* positions, int n, int T, int W, int f32, hipStream_t s);
+int k8s_shift_save(void* state, const void* h, const int* cu_q, const int* seq_slots, const int* positions, int nseq,
+                   int W, int f32, hipStream_t s);
+int k8s_wkv_max_dim();
+int k8s_wkv_scan(void* out, const void* r, const void* k, const void* v, const void* g, long ld, const float* z,
+                 const void* w0, const void* u, const void* lnw, float* state, const int* cu_q, const int* seq_slots,
+                 const int* positions, int nseq, int H, int D, float eps, int f32, hipStream_t s);
+int k8s_latent_kv_write(void* cache, const void* dkv, const void* normw, void* q, const float* cos_sin,
+                        const int* positions, const int* slot_mapping, int T, int C, int R, int H, int Dn, int dims,
+                        float eps, int f32, hipStream_t s);
+int k8s_latent_attention(void* out, const void* q_abs, const void* q, const void* cache, const int* block_tables,
+                         int max_blocks, const int* tok_seq, const int* positions, int T, int C, int R, int H, int Dn,
+                         int window, float scale, int bs, int f32, hipStream_t s);
+int k8s_moe_route(int* idx, float* w, const float* logits, int ld, int T, int E, int top, float scale, hipStream_t s);
+int k8s_moe_align(int* sorted_tok, int* pos_of_pair, int* seg, int* tiles, int ntiles, const int* topk_idx, int P,
+                  int top, int E, int BM, hipStream_t s);
+int k8s_moe_combine(void* z, const void* D, const int* pos, const float* w, const void* shared, const float* logits,
+                    int ld, int sg_col, int T, int W, int top, int f32, hipStream_t s);
 int k8s_pgemm_num_configs();
 int k8s_pgemm_config(int cfg, int* bp, int* bq, int* lds_bytes);
 int k8s_pgemm_plan(int M, int N_out, int K, int epi, int fp8, int cfg, int splits, int* nwg, long long* ws_elems,
@@ -348,6 +374,67 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
   m.def("hash_init", [](uintptr_t out, int rows, int cols, long long gcols, long long row0, long long col0,
                         uint32_t seed, uint32_t tid, float scale, float shift, int64_t s) {
     check(k8s_hash_init(P(out), rows, cols, gcols, row0, col0, seed, tid, scale, shift, S(s)), "hash_init");
+  });
+
+  // fp32 residual stream, recurrent / latent mixers, mixture of experts (stream32.hip, mixers.hip, moe.hip)
+  m.def("embed_rows", [](uintptr_t out, uintptr_t ids, uintptr_t table, int T, int W, int vocab, int f32, int64_t s) {
+    check(k8s_embed_rows(P<float>(out), P<int>(ids), P(table), T, W, vocab, f32, S(s)), "embed_rows");
+  });
+  m.def("resnorm", [](uintptr_t x, uintptr_t branch, float mult, uintptr_t rowvec, uintptr_t w, float offset, float eps,
+                      uintptr_t out, int T, int W, int f32, int64_t s) {
+    check(k8s_resnorm(P<float>(x), P(branch), mult, P(rowvec), P(w), offset, eps, P(out), T, W, f32, S(s)), "resnorm");
+  });
+  m.def("act", [](uintptr_t out, uintptr_t x, int T, int F, int kind, float limit, float alpha, int f32, int64_t s) {
+    check(k8s_act(P(out), P(x), T, F, kind, limit, alpha, f32, S(s)), "act");
+  });
+  m.def("gemm_any", [](uintptr_t C, uintptr_t A, uintptr_t W, int M, int N, int K, long lda, long ldw, long ldc,
+                       int batch, long sA, long sW, long sC, uintptr_t a_rows, uintptr_t tiles, int ntiles, int in_f32,
+                       int out_f32, int64_t s) {
+    check(k8s_gemm_any(P(C), P(A), P(W), M, N, K, lda, ldw, ldc, batch, sA, sW, sC, P<int>(a_rows), P<int>(tiles),
+                       ntiles, in_f32, out_f32, S(s)), "gemm_any");
+  });
+  m.def("token_shift", [](uintptr_t out, uintptr_t h, uintptr_t mu, uintptr_t state, uintptr_t cu_q, uintptr_t tok_seq,
+                          uintptr_t seq_slots, uintptr_t positions, int n, int T, int W, int f32, int64_t s) {
+    check(k8s_token_shift(P(out), P(h), P(mu), P(state), P<int>(cu_q), P<int>(tok_seq), P<int>(seq_slots),
+                          P<int>(positions), n, T, W, f32, S(s)), "token_shift");
+  });
+  m.def("shift_save", [](uintptr_t state, uintptr_t h, uintptr_t cu_q, uintptr_t seq_slots, uintptr_t positions,
+                         int nseq, int W, int f32, int64_t s) {
+    check(k8s_shift_save(P(state), P(h), P<int>(cu_q), P<int>(seq_slots), P<int>(positions), nseq, W, f32, S(s)),
+          "shift_save");
+  });
+  m.def("wkv_max_dim", []() { return k8s_wkv_max_dim(); });
+  m.def("wkv_scan", [](uintptr_t out, uintptr_t r, uintptr_t k, uintptr_t v, uintptr_t g, long ld, uintptr_t z,
+                       uintptr_t w0, uintptr_t u, uintptr_t lnw, uintptr_t state, uintptr_t cu_q, uintptr_t seq_slots,
+                       uintptr_t positions, int nseq, int H, int D, float eps, int f32, int64_t s) {
+    check(k8s_wkv_scan(P(out), P(r), P(k), P(v), P(g), ld, P<float>(z), P(w0), P(u), P(lnw), P<float>(state),
+                       P<int>(cu_q), P<int>(seq_slots), P<int>(positions), nseq, H, D, eps, f32, S(s)), "wkv_scan");
+  });
+  m.def("latent_kv_write", [](uintptr_t cache, uintptr_t dkv, uintptr_t normw, uintptr_t q, uintptr_t cos_sin,
+                              uintptr_t positions, uintptr_t slots, int T, int C, int R, int H, int Dn, int dims,
+                              float eps, int f32, int64_t s) {
+    check(k8s_latent_kv_write(P(cache), P(dkv), P(normw), P(q), P<float>(cos_sin), P<int>(positions), P<int>(slots), T,
+                              C, R, H, Dn, dims, eps, f32, S(s)), "latent_kv_write");
+  });
+  m.def("latent_attention", [](uintptr_t out, uintptr_t q_abs, uintptr_t q, uintptr_t cache, uintptr_t bt,
+                               int max_blocks, uintptr_t tok_seq, uintptr_t positions, int T, int C, int R, int H,
+                               int Dn, int window, float scale, int bs, int f32, int64_t s) {
+    check(k8s_latent_attention(P(out), P(q_abs), P(q), P(cache), P<int>(bt), max_blocks, P<int>(tok_seq),
+                               P<int>(positions), T, C, R, H, Dn, window, scale, bs, f32, S(s)), "latent_attention");
+  });
+  m.def("moe_route", [](uintptr_t idx, uintptr_t w, uintptr_t logits, int ld, int T, int E, int top, float scale,
+                        int64_t s) {
+    check(k8s_moe_route(P<int>(idx), P<float>(w), P<float>(logits), ld, T, E, top, scale, S(s)), "moe_route");
+  });
+  m.def("moe_align", [](uintptr_t sorted_tok, uintptr_t pos, uintptr_t seg, uintptr_t tiles, int ntiles,
+                        uintptr_t topk_idx, int P_, int top, int E, int BM, int64_t s) {
+    check(k8s_moe_align(P<int>(sorted_tok), P<int>(pos), P<int>(seg), P<int>(tiles), ntiles, P<int>(topk_idx), P_, top,
+                        E, BM, S(s)), "moe_align");
+  });
+  m.def("moe_combine", [](uintptr_t z, uintptr_t D, uintptr_t pos, uintptr_t w, uintptr_t shared, uintptr_t logits,
+                          int ld, int sg_col, int T, int W, int top, int f32, int64_t s) {
+    check(k8s_moe_combine(P(z), P(D), P<int>(pos), P<float>(w), P(shared), P<float>(logits), ld, sg_col, T, W, top,
+                          f32, S(s)), "moe_combine");
   });
 
   m.def("mgemm_configs", []() {

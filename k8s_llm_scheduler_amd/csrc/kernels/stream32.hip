@@ -1,0 +1,213 @@
+// fp32 residual stream: embedding rows, fused residual-add + RMS norm, gated activations, and a GEMM for any shape.
+//
+// Models whose residual sum lives in fp32 keep x as [T, W] floats; every branch output (bf16, or fp32 in the all-fp32
+// mode) is added in fp32 by the norm that follows it, so the add costs no extra pass.  All kernels take the
+// activation / weight element type as a template parameter: bf16 storage or true fp32.
+#include "common.h"
+
+namespace k8sllm {
+
+// out[t, :] = float(table[ids[t], :])
+template <typename TA>
+__global__ void embed_rows_kernel(float* __restrict__ out, const int* __restrict__ ids, const TA* __restrict__ table,
+                                  int W, int vocab) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  for (int i = threadIdx.x; i < W; i += blockDim.x) out[(size_t)t * W + i] = ldf(table, (size_t)id * W + i);
+}
+
+// x[t] += mult * branch[t] + rowvec (each optional), stored back in fp32; then (w != null)
+// out[t] = x[t] / sqrt(mean(x[t]^2) + eps) * (offset + w).  One workgroup per row; the row stays in registers / LDS
+// between the add and the norm.
+template <typename TA>
+__global__ __launch_bounds__(256) void resnorm_kernel(float* __restrict__ x, const TA* __restrict__ branch, float mult,
+                                                      const TA* __restrict__ rowvec, const TA* __restrict__ w,
+                                                      float offset, float eps, TA* __restrict__ out, int W) {
+  __shared__ float red[16];
+  const size_t base = (size_t)blockIdx.x * W;
+  float ss = 0.f;
+  const bool upd = branch != nullptr || rowvec != nullptr;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float v = x[base + i];
+    if (branch != nullptr) v += mult * ldf(branch, base + i);
+    if (rowvec != nullptr) v += ldf(rowvec, i);
+    if (upd) x[base + i] = v;
+    ss += v * v;
+  }
+  if (w == nullptr) return;
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)W + eps);
+  for (int i = threadIdx.x; i < W; i += blockDim.x)
+    stf(out, base + i, x[base + i] * inv * (offset + ldf(w, i)));
+}
+
+// kinds: 0 gelu_tanh(g) * u, 1 g' * sigmoid(alpha g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, +-limit)
+// (limit <= 0: no clamp) -- both read [T, 2F] = [gate | up]; 2 tanh, 3 silu: elementwise on [T, F].
+template <typename TA>
+__global__ void act_kernel(TA* __restrict__ out, const TA* __restrict__ x, int T, int F, int kind, float limit,
+                           float alpha) {
+  const size_t n = (size_t)T * F;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = i / F, c = i - t * F;
+    float y;
+    if (kind >= 2) {
+      const float v = ldf(x, i);
+      y = kind == 2 ? tanhf(v) : v / (1.f + expf(-v));
+    } else {
+      float g = ldf(x, t * 2 * F + c), u = ldf(x, t * 2 * F + F + c);
+      if (kind == 0) {
+        y = 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
+      } else {
+        if (limit > 0.f) {
+          g = fminf(g, limit);
+          u = fminf(fmaxf(u, -limit), limit);
+        }
+        y = g / (1.f + expf(-alpha * g)) * (u + 1.f);
+      }
+    }
+    stf(out, i, y);
+  }
+}
+
+// C = A W^T for any M, N, K and any row strides: 64 x 64 output tile per workgroup, 16-deep k steps staged through LDS
+// as fp32, 4 x 4 outputs per thread, fp32 FMA accumulation in k order (a row's result does not depend on which rows
+// share its tile).  Three forms:
+//   plain / strided-batched: blockIdx.z = batch g, operands offset by g * (sA, sW, sC);
+//   row gather: A row r is A[a_rows[r]];
+//   grouped: tiles[y] = (group, first row, rows) lists the row tiles of variable-size groups over one compact row
+//   space (a mixture-of-experts' sorted tokens); group g uses W + g * sW; tiles with group < 0 are padding.
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void gemm_any_kernel(TO* __restrict__ C, const TI* __restrict__ A,
+                                                       const TI* __restrict__ Wt, int M, int N, int K, long lda,
+                                                       long ldw, long ldc, long sA, long sW, long sC,
+                                                       const int* __restrict__ a_rows, const int* __restrict__ tiles) {
+  constexpr int BM = 64, BN = 64, BK = 16, LD = BM + 4;
+  __shared__ __attribute__((aligned(16))) float As[BK][LD];
+  __shared__ __attribute__((aligned(16))) float Ws[BK][LD];
+  int row0, rows;
+  if (tiles != nullptr) {
+    const int g = tiles[3 * blockIdx.y];
+    if (g < 0) return;
+    row0 = tiles[3 * blockIdx.y + 1];
+    rows = tiles[3 * blockIdx.y + 2];
+    Wt += (size_t)g * sW;
+  } else {
+    row0 = blockIdx.y * BM;
+    rows = min(BM, M - row0);
+    A += (size_t)blockIdx.z * sA;
+    Wt += (size_t)blockIdx.z * sW;
+    C += (size_t)blockIdx.z * sC;
+  }
+  const int col0 = blockIdx.x * BN;
+  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+  const int kk = tid & 15, r_l = tid >> 4;          // loader: k index, first of 4 rows (r_l + 16 i)
+  size_t a_off[4], w_off[4];
+  bool a_ok[4], w_ok[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = r_l + 16 * i;
+    a_ok[i] = r < rows;
+    const int gr = a_ok[i] ? (a_rows != nullptr ? a_rows[row0 + r] : row0 + r) : 0;
+    a_off[i] = (size_t)gr * lda;
+    w_ok[i] = col0 + r < N;
+    w_off[i] = (size_t)(w_ok[i] ? col0 + r : 0) * ldw;
+  }
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    const bool kin = k0 + kk < K;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      As[kk][r_l + 16 * i] = (kin && a_ok[i]) ? ldf(A, a_off[i] + k0 + kk) : 0.f;
+      Ws[kk][r_l + 16 * i] = (kin && w_ok[i]) ? ldf(Wt, w_off[i] + k0 + kk) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < BK; ++k) {
+      const f32x4 a = *reinterpret_cast<const f32x4*>(&As[k][ty * 4]);
+      const f32x4 b = *reinterpret_cast<const f32x4*>(&Ws[k][tx * 4]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = ty * 4 + i;
+    if (r >= rows) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = col0 + tx * 4 + j;
+      if (c < N) stf(C, (size_t)(row0 + r) * ldc + c, acc[i][j]);
+    }
+  }
+}
+
+}  // namespace k8sllm
+
+using namespace k8sllm;
+
+extern "C" int k8s_embed_rows(float* out, const int* ids, const void* table, int T, int W, int vocab, int f32,
+                              hipStream_t s) {
+  if (T <= 0) return 0;
+  if (W <= 0 || vocab <= 0) return -1;
+  if (f32) embed_rows_kernel<float><<<T, 256, 0, s>>>(out, ids, (const float*)table, W, vocab);
+  else embed_rows_kernel<bf16_t><<<T, 256, 0, s>>>(out, ids, (const bf16_t*)table, W, vocab);
+  return (int)hipGetLastError();
+}
+
+extern "C" int k8s_resnorm(float* x, const void* branch, float mult, const void* rowvec, const void* w, float offset,
+                           float eps, void* out, int T, int W, int f32, hipStream_t s) {
+  if (T <= 0) return 0;
+  if (W <= 0 || (w != nullptr && out == nullptr)) return -1;
+  if (f32)
+    resnorm_kernel<float><<<T, 256, 0, s>>>(x, (const float*)branch, mult, (const float*)rowvec, (const float*)w,
+                                            offset, eps, (float*)out, W);
+  else
+    resnorm_kernel<bf16_t><<<T, 256, 0, s>>>(x, (const bf16_t*)branch, mult, (const bf16_t*)rowvec, (const bf16_t*)w,
+                                             offset, eps, (bf16_t*)out, W);
+  return (int)hipGetLastError();
+}
+
+extern "C" int k8s_act(void* out, const void* x, int T, int F, int kind, float limit, float alpha, int f32,
+                       hipStream_t s) {
+  if (T <= 0 || F <= 0) return 0;
+  if (kind < 0 || kind > 3) return -1;
+  const size_t n = (size_t)T * F;
+  const int blocks = (int)((n + 255) / 256 > 4096 ? 4096 : (n + 255) / 256);
+  if (f32) act_kernel<float><<<blocks, 256, 0, s>>>((float*)out, (const float*)x, T, F, kind, limit, alpha);
+  else act_kernel<bf16_t><<<blocks, 256, 0, s>>>((bf16_t*)out, (const bf16_t*)x, T, F, kind, limit, alpha);
+  return (int)hipGetLastError();
+}
+
+extern "C" int k8s_gemm_any(void* C, const void* A, const void* W, int M, int N, int K, long lda, long ldw, long ldc,
+                            int batch, long sA, long sW, long sC, const int* a_rows, const int* tiles, int ntiles,
+                            int in_f32, int out_f32, hipStream_t s) {
+  if (N <= 0 || K <= 0 || batch <= 0) return -1;
+  int gy;
+  if (tiles != nullptr) {
+    if (ntiles <= 0) return 0;
+    gy = ntiles;
+    batch = 1;
+  } else {
+    if (M <= 0) return 0;
+    gy = (M + 63) / 64;
+  }
+  if (gy > 65535 || batch > 65535) return -2;
+  const dim3 grid((N + 63) / 64, gy, batch);
+#define K8S_GA(TI, TO) \
+  gemm_any_kernel<TI, TO><<<grid, 256, 0, s>>>((TO*)C, (const TI*)A, (const TI*)W, M, N, K, lda, ldw, ldc, sA, sW, sC, \
+                                               a_rows, tiles)
+  if (in_f32 && out_f32) K8S_GA(float, float);
+  else if (in_f32) K8S_GA(float, bf16_t);
+  else if (out_f32) K8S_GA(bf16_t, float);
+  else K8S_GA(bf16_t, bf16_t);
+#undef K8S_GA
+  return (int)hipGetLastError();
+}

@@ -87,33 +87,46 @@ def build_engine(preset: str = "llama-3.3-70b", *, tp=None, device: Optional[str
                  max_model_len: int = 16384, max_prefill_tokens: int = 8192, cuda_graphs: bool = True,
                  prefix_caching: bool = True, decode_chunk: int = 4, metrics=None, capture: bool = True, control=None,
                  weight_dtype: str = "bf16", capture_nucleus: bool = False, speculative_tokens: int = 0,
-                 watchdog_s: float = 60.0, on_unrecoverable: str = "stay", mixed_step_rows: int = 256):
-    """Model + tokenizer + engine on this rank's GPU (or CPU when no GPU is present).
+                 watchdog_s: float = 60.0, on_unrecoverable: str = "stay", mixed_step_rows: int = 256,
+                 dtype: str = "bfloat16"):
+    """Model + tokenizer + engine on this rank's GPU (or CPU when no GPU is present).  The model class follows the
+    preset's / checkpoint's configuration (``models.load_config``, ``models.model_class``).
     ``weight_dtype``: "bf16" or "fp8" (row-scaled e4m3 projection weights).  ``capture_nucleus``:
-    decode graphs with the top-p sampler passes too (serving with top_p < 1)."""
+    decode graphs with the top-p sampler passes too (serving with top_p < 1).  ``dtype``: "bfloat16", or "float32" for
+    the models that run in true fp32."""
     import torch
 
-    from ..models.config import get_config
-    from ..models.llama import LlamaModel
+    from ..models import load_config, model_class
     from ..parallel import TPGroup
     from .engine import LLMEngine
+    from .tokenizer import IdTokenizer
 
     tp = tp or TPGroup()
     if device is None:
         device = f"cuda:{torch.cuda.current_device()}" if torch.cuda.is_available() else "cpu"
-    cfg = get_config(weights or preset) if weights else get_config(preset)
+    cfg = load_config(weights or preset)
+    Model = model_class(cfg)
+    kw = {}
+    if dtype not in ("bfloat16", "bf16"):
+        if dtype not in ("float32", "fp32") or not getattr(Model, "stateful", False):
+            raise ValueError(f"{cfg.name}: dtype {dtype!r} is not supported by {Model.__name__}")
+        kw["dtype"] = torch.float32
     from .. import ops
 
     if device.startswith("cuda") and ops.GEMM_BACKEND == "library":
         _load_gemm_table()
     t0 = time.perf_counter()
-    model = LlamaModel(cfg, tp, device=device, seed=seed, weights=weights, max_model_len=max_model_len,
-                       weight_dtype=weight_dtype)
+    model = Model(cfg, tp, device=device, seed=seed, weights=weights, max_model_len=max_model_len,
+                  weight_dtype=weight_dtype, **kw)
     if device.startswith("cuda"):
         torch.cuda.synchronize()
     log.info(f" Model {cfg.name} ready on {device} (tp {tp.rank}/{tp.world}, "
              f"{model.weight_bytes() / 1e9:.1f} GB weights, {time.perf_counter() - t0:.1f}s)")
-    tok = Tokenizer(resolve_tokenizer(weights, tokenizer), model_vocab=cfg.vocab)
+    if tokenizer == "ids" or (tokenizer is None and getattr(cfg, "token_ids_only", False)
+                              and not (weights and (Path(weights) / "tokenizer.json").is_file())):
+        tok = IdTokenizer(cfg.vocab)
+    else:
+        tok = Tokenizer(resolve_tokenizer(weights, tokenizer), model_vocab=cfg.vocab)
     eng = LLMEngine(model, tok, max_batch=max_batch, block_size=block_size, num_blocks=num_blocks,
                     kv_cache_gb=kv_cache_gb, kv_cache_fraction=kv_cache_fraction, max_model_len=max_model_len,
                     max_prefill_tokens=max_prefill_tokens, cuda_graphs=cuda_graphs, prefix_caching=prefix_caching,
@@ -121,7 +134,7 @@ def build_engine(preset: str = "llama-3.3-70b", *, tp=None, device: Optional[str
                     capture_nucleus=capture_nucleus, speculative_tokens=speculative_tokens, watchdog_s=watchdog_s,
                     on_unrecoverable=on_unrecoverable, mixed_step_rows=mixed_step_rows)
     if device.startswith("cuda"):
-        warm_gemms(model)
+        model.warm() if hasattr(model, "warm") else warm_gemms(model)
     if capture and eng.use_graphs:
         t1 = time.perf_counter()
         eng.capture_graphs()

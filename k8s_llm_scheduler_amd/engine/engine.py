@@ -56,9 +56,10 @@ from .graphs import GraphCaptureMixin
 from .recovery import RecoveryMixin
 from .serving import ServingMixin
 from .speculative import SpeculativeMixin
+from .replay import ReplayMixin
 
 
-class LLMEngine(GraphCaptureMixin, RecoveryMixin, SpeculativeMixin, ServingMixin):
+class LLMEngine(GraphCaptureMixin, RecoveryMixin, SpeculativeMixin, ServingMixin, ReplayMixin):
     def __init__(self, model: LlamaModel, tokenizer: Tokenizer, *, max_batch: int = 64, block_size: int = 16,
                  num_blocks: Optional[int] = None, kv_cache_gb: float = 0.0, kv_cache_fraction: float = 0.85,
                  max_model_len: Optional[int] = None, max_prefill_tokens: int = 8192, cuda_graphs: bool = True,
@@ -109,6 +110,12 @@ class LLMEngine(GraphCaptureMixin, RecoveryMixin, SpeculativeMixin, ServingMixin
             control.start_monitor()
         # prompt-lookup speculative decoding (_spec_decode): drafted tokens per step, 0 = off
         self.speculative_tokens = max(0, int(speculative_tokens))
+        # a model with per-slot recurrent state (model.stateful): a verify forward cannot be rolled back and a cached
+        # prefix holds no state, so speculative decoding and prefix caching are off; the model gets each sequence's slot
+        self.stateful = bool(getattr(model, "stateful", False))
+        if self.stateful:
+            self.speculative_tokens = 0
+            prefix_caching = False
         if self.speculative_tokens:
             # the verify steps emit tokens on the host without advancing the sampler's device stop state (JSON
             # depth, done flag), so a later one-token decode would see a stale brace depth and could end an answer
@@ -153,6 +160,8 @@ class LLMEngine(GraphCaptureMixin, RecoveryMixin, SpeculativeMixin, ServingMixin
         self.num_blocks = num_blocks
         # one extra block past the allocator's range: the K/V sink of prefill-graph padding tokens
         model.allocate_kv(num_blocks + 1, block_size)
+        if self.stateful:
+            model.allocate_state(max_batch)
         self.scratch_slot = num_blocks * block_size
         self.prefix_caching = prefix_caching
         self._share_deferred = False
@@ -398,6 +407,23 @@ class LLMEngine(GraphCaptureMixin, RecoveryMixin, SpeculativeMixin, ServingMixin
         dst = self._dev(list(range(dst_block * bs, dst_block * bs + n)), torch.long)
         kv.index_copy_(2, dst, kv.index_select(2, src))
 
+    def _chunk_inputs(self, chunk) -> tuple:
+        """Host-side inputs of one varlen forward over ``chunk`` = [(request, start, end)]: token ids, positions and
+        cache slots of every token, the sequences' query offsets, context lengths after the chunk, each sequence's
+        last row, and the block tables."""
+        bs = self.block_size
+        ids, pos, slots, cu, ctx, last = [], [], [], [0], [], []
+        bt = torch.zeros(len(chunk), self.max_blocks_per_seq, dtype=torch.int32)
+        for i, (r, s, e) in enumerate(chunk):
+            ids += r.prompt_ids[s:e]
+            pos += range(s, e)
+            slots += [r.blocks[p // bs] * bs + p % bs for p in range(s, e)]
+            cu.append(cu[-1] + (e - s))
+            ctx.append(e)
+            last.append(cu[-1] - 1)
+            bt[i, :len(r.blocks)] = torch.tensor(r.blocks, dtype=torch.int32)
+        return ids, pos, slots, cu, ctx, last, bt
+
     def _prefill(self) -> None:
         if not self.prefilling:
             return
@@ -423,16 +449,7 @@ class LLMEngine(GraphCaptureMixin, RecoveryMixin, SpeculativeMixin, ServingMixin
             chunk.append((r, r.computed, r.computed + n))
             budget -= n
         bs = self.block_size
-        ids, pos, slots, cu, ctx, last = [], [], [], [0], [], []
-        bt = torch.zeros(len(chunk), self.max_blocks_per_seq, dtype=torch.int32)
-        for i, (r, s, e) in enumerate(chunk):
-            ids += r.prompt_ids[s:e]
-            pos += range(s, e)
-            slots += [r.blocks[p // bs] * bs + p % bs for p in range(s, e)]
-            cu.append(cu[-1] + (e - s))
-            ctx.append(e)
-            last.append(cu[-1] - 1)
-            bt[i, :len(r.blocks)] = torch.tensor(r.blocks, dtype=torch.int32)
+        ids, pos, slots, cu, ctx, last, bt = self._chunk_inputs(chunk)
         dev = self.device
         t = self._dev
         t0 = time.perf_counter()
@@ -467,7 +484,8 @@ class LLMEngine(GraphCaptureMixin, RecoveryMixin, SpeculativeMixin, ServingMixin
             bt_t = torch.cat([self._dev(bt), self.s_bt.index_select(0, d)])
             last_t = t(last + [n_p + k for k in range(len(dec))])
             logits = self.model.forward_prefill(ids_t, pos_t, slot_t, t(cu_all), ctx_t, bt_t,
-                                                max(e - s for _, s, e in chunk), last_t)
+                                                max(e - s for _, s, e in chunk), last_t,
+                                                **self._state_kw([r.slot for r, _, _ in chunk] + dec))
             # the decode rows' tokens: the decode graphs' sampler (same counters, same stop detection), with the
             # state of each row's slot updated in place
             ld = logits[:, len(chunk):].contiguous()
@@ -492,7 +510,8 @@ class LLMEngine(GraphCaptureMixin, RecoveryMixin, SpeculativeMixin, ServingMixin
                 split = (T0, halves[0], halves[1])
                 self.stats["prefill_overlap_chunks"] += 1
             logits = self.model.forward_prefill(t(ids), t(pos), t(slots), t(cu), t(ctx), bt_d,
-                                                max(e - s for _, s, e in chunk), t(last), split=split)
+                                                max(e - s for _, s, e in chunk), t(last), split=split,
+                                                **self._state_kw([r.slot for r, _, _ in chunk]))
         self.stats["prefill_tokens"] += len(ids)
         self.stats["prefill_steps"] = self.stats.get("prefill_steps", 0) + 1
         if self._trace_steps:
@@ -560,6 +579,10 @@ class LLMEngine(GraphCaptureMixin, RecoveryMixin, SpeculativeMixin, ServingMixin
                 self._account_prefill()
         else:
             self.stats["prefill_time"] += time.perf_counter() - t0
+
+    def _state_kw(self, slots: Sequence[int]) -> dict:
+        """forward_prefill's extra argument for a stateful model: the state slot of every sequence of the batch."""
+        return {"seq_slots": self._dev(list(slots))} if self.stateful else {}
 
     def _account_prefill(self) -> None:
         """Add the GPU time of completed prefills to stats["prefill_time"] (after a device wait)."""

@@ -149,6 +149,8 @@ class GraphCaptureMixin:
         Multi-rank engines capture only the buckets whose collectives all stay on xGMI
         (``_prefill_bucket_capturable``); ``K8S_PREFILL_GRAPHS=1`` captures every bucket (RCCL included)."""
         env = os.environ.get("K8S_PREFILL_GRAPHS", "")
+        if not getattr(self.model, "prefill_graphs", True):
+            return False     # (a stateful model's chunk carries its sequence's state slot: not a padded static input)
         return env != "0" and self.use_graphs and PREFILL_GRAPH_BUCKETS[-1] <= self.max_prefill_tokens
 
     def _decode_bucket_capturable(self, B: int) -> bool:

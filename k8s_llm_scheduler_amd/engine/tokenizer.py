@@ -62,3 +62,47 @@ class Tokenizer:
             ids += [sh] + self.encode(role) + [eh] + self.encode("\n\n" + content.strip()) + [eot]
         ids += [sh] + self.encode("assistant") + [eh] + self.encode("\n\n")
         return ids
+
+
+class _IdVocab:
+    """The part of the ``tokenizers`` interface the engine's stop tables read, for a vocabulary without text."""
+
+    def __init__(self, n: int):
+        self.n = n
+
+    def get_vocab_size(self) -> int:
+        return self.n
+
+    def get_vocab(self) -> dict:
+        return {}
+
+    def decode_batch(self, rows, skip_special_tokens: bool = True) -> List[str]:
+        return ["" for _ in rows]
+
+
+class IdTokenizer:
+    """Tokenizer of a model served by token ids (a checkpoint without tokenizer.json whose vocabulary the built-in
+    synthetic one does not fit): text is a whitespace-separated list of ids; no end-of-sequence or brace tokens, so a
+    request ends at max_tokens or one of its own stop_token_ids."""
+
+    synthetic = True
+
+    def __init__(self, model_vocab: int):
+        self.model_vocab = model_vocab
+        self._tok = _IdVocab(model_vocab)
+        self.special: dict = {}
+        self.bos_id = 0
+        self.eot_id = -1
+        self.eos_ids: set = set()
+
+    def encode(self, text: str) -> List[int]:
+        ids = [int(t) for t in text.split()]
+        if any(i < 0 or i >= self.model_vocab for i in ids):
+            raise ValueError("token id outside the vocabulary")
+        return ids
+
+    def decode(self, ids: Sequence[int]) -> str:
+        return " ".join(str(int(i)) for i in ids)
+
+    def chat_ids(self, system: str, user: str, knowledge_dates: bool = True) -> List[int]:
+        return self.encode(system) + self.encode(user)

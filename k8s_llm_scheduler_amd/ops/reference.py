@@ -480,3 +480,198 @@ def write_token_stop(s: int, tok: int, tokens, ctx_inc, hist, steps, stop) -> No
     ctx_inc[s] = 0 if fin else int(ctx_inc[s]) + 1
     if fin:
         stop["done"][s] = 1
+
+
+# ----------------------------------------------------------------------------- fp32 residual stream, gated activations
+ACT_GELU_TANH, ACT_SWISH_CLAMP, ACT_TANH, ACT_SILU = 0, 1, 2, 3
+
+
+def embed_rows(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """fp32 rows of the embedding table (the residual stream starts in fp32)."""
+    return table.index_select(0, ids.long()).float()
+
+
+def resnorm(x: torch.Tensor, branch, mult: float, rowvec, w, offset: float, eps: float, out_dtype):
+    """x (fp32, in place) += mult * branch + rowvec; returns x / sqrt(mean(x^2) + eps) * (offset + w) or None."""
+    if branch is not None:
+        x.add_(branch.float() * mult)
+    if rowvec is not None:
+        x.add_(rowvec.float())
+    if w is None:
+        return None
+    y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * (offset + w.float())
+    return y.to(out_dtype)
+
+
+def act(x: torch.Tensor, kind: int, limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
+    """Gated kinds take [T, 2F] = [gate | up] and return [T, F]; ACT_TANH / ACT_SILU are elementwise."""
+    if kind in (ACT_TANH, ACT_SILU):
+        f = x.float()
+        return (torch.tanh(f) if kind == ACT_TANH else f * torch.sigmoid(f)).to(x.dtype)
+    F = x.shape[-1] // 2
+    g, u = x[..., :F].float(), x[..., F:].float()
+    if kind == ACT_GELU_TANH:
+        y = 0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g * g * g))) * u
+    else:
+        if limit > 0:
+            g = g.clamp(max=limit)
+            u = u.clamp(-limit, limit)
+        y = g * torch.sigmoid(alpha * g) * (u + 1.0)
+    return y.to(x.dtype)
+
+
+def gemm_any(a: torch.Tensor, w: torch.Tensor, out_dtype, a_rows=None, tiles=None, seg=None) -> torch.Tensor:
+    """a [M, K] @ w [N, K]^T, or batched a [G, M, K] (any strides) @ w [G, N, K]^T -> [G, M, N]; grouped
+    (``seg`` [G + 1] row offsets into the gathered rows ``a[a_rows]``): rows seg[g] .. seg[g + 1] use w[g]."""
+    if seg is not None:
+        rows = a.index_select(0, a_rows.long()).float() if a_rows is not None else a.float()
+        out = torch.zeros(rows.shape[0], w.shape[1], dtype=torch.float32)
+        s = seg.tolist()
+        for g in range(len(s) - 1):
+            if s[g + 1] > s[g]:
+                out[s[g]:s[g + 1]] = rows[s[g]:s[g + 1]] @ w[g].float().T
+        return out.to(out_dtype)
+    return (a.float() @ w.float().transpose(-1, -2)).to(out_dtype)
+
+
+# ----------------------------------------------------------------------------- recurrent mixer (token shift + wkv)
+def token_shift(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor, seq_slots: torch.Tensor,
+                positions: torch.Tensor) -> torch.Tensor:
+    """out[s, t] = h[t] + (prev[t] - h[t]) * mu[s]; prev is the previous token of the same sequence: h[t - 1]
+    inside a portion, the slot's saved row at a portion's start, zeros at position 0.  Rows with position < 0 are
+    skipped (zeros).  [n, T, W]."""
+    T, W = h.shape
+    hf = h.float()
+    prev = torch.zeros(T, W)
+    cu = cu_q.tolist()
+    for s in range(len(cu) - 1):
+        a, b = cu[s], cu[s + 1]
+        if b <= a or int(positions[a]) < 0:
+            continue
+        prev[a + 1:b] = hf[a:b - 1]
+        if int(positions[a]) > 0:
+            prev[a] = state[int(seq_slots[s])].float()
+    out = hf.unsqueeze(0) + (prev - hf).unsqueeze(0) * mu.float().unsqueeze(1)
+    return out.to(h.dtype)
+
+
+def shift_save(state: torch.Tensor, h: torch.Tensor, cu_q: torch.Tensor, seq_slots: torch.Tensor,
+               positions: torch.Tensor) -> None:
+    cu = cu_q.tolist()
+    for s in range(len(cu) - 1):
+        a, b = cu[s], cu[s + 1]
+        if b > a and int(positions[a]) >= 0:
+            state[int(seq_slots[s])] = h[b - 1]
+
+
+def wkv_scan(r, k, v, g, z, w0, u, lnw, state, cu_q, seq_slots, positions, H: int, D: int, eps: float, out_dtype):
+    """Per head: o_t = (S + diag(u) k_t v_t^T)^T r_t, S <- diag(w_t) S + k_t v_t^T with w = exp(-exp(z + w0));
+    the head's o / rms(o) * lnw * silu(g).  ``state`` [slots, H, D, D] fp32 carries S between calls (zero at
+    position 0)."""
+    T = r.shape[0]
+    out = torch.zeros(T, H * D)
+    w = torch.exp(-torch.exp(z.float() + w0.float()))
+    rf, kf, vf, gf = (t.float().view(T, H, D) for t in (r, k, v, g))
+    w = w.view(T, H, D)
+    uf = u.float().view(H, D)
+    cu = cu_q.tolist()
+    for s in range(len(cu) - 1):
+        a, b = cu[s], cu[s + 1]
+        if b <= a or int(positions[a]) < 0:
+            continue
+        slot = int(seq_slots[s])
+        S = torch.zeros(H, D, D) if int(positions[a]) == 0 else state[slot].clone()
+        for t in range(a, b):
+            kv = kf[t].unsqueeze(2) * vf[t].unsqueeze(1)                   # [H, D, D]
+            o = torch.einsum("hi,hij->hj", rf[t], S + uf.unsqueeze(2) * kv)
+            S = w[t].unsqueeze(2) * S + kv
+            o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+            out[t] = o.reshape(-1)
+        state[slot] = S
+    g2 = gf.reshape(T, H * D)
+    return (out * lnw.float() * g2 * torch.sigmoid(g2)).to(out_dtype)
+
+
+# ----------------------------------------------------------------------------- latent attention
+def latent_kv_write(cache, dkv, normw, q, cos_sin, positions, slot_mapping, C: int, R: int, H: int, Dn: int,
+                    rot_dims: int, eps: float) -> None:
+    """cache[slot] = [rms(dkv[:C]) * normw | rope(dkv[C:])]; q's rotated part ([T, H, Dn + R], last R of each head)
+    is rotated in place.  Rows with a negative slot are not written."""
+    T = dkv.shape[0]
+    d = dkv.float()
+    c = d[:, :C] * torch.rsqrt(d[:, :C].pow(2).mean(-1, keepdim=True) + eps) * normw.float()
+    half = rot_dims // 2
+    cs = cos_sin[positions.long().clamp(min=0)]
+    cos, sin = cs[:, :half], cs[:, half:]
+
+    def rot(x, cos, sin):
+        a, b = x[..., :half], x[..., half:rot_dims]
+        return torch.cat([a * cos - b * sin, b * cos + a * sin, x[..., rot_dims:]], -1)
+
+    kr = rot(d[:, C:], cos, sin)
+    row = torch.cat([c, kr], -1).to(cache.dtype)
+    ok = slot_mapping >= 0
+    cache[slot_mapping[ok].long()] = row[ok]
+    qv = q.view(T, H, Dn + R)
+    qv[..., Dn:] = rot(qv[..., Dn:].float(), cos.unsqueeze(1), sin.unsqueeze(1)).to(q.dtype)
+
+
+def latent_attention(q_abs, q, cache, block_tables, tok_seq, positions, C: int, R: int, H: int, Dn: int,
+                     window: int, scale: float, block_size: int, out_dtype):
+    """Token t of sequence tok_seq[t] at position p attends the cached rows of positions max(0, p - window + 1) .. p
+    (window <= 0: all): score = (q_abs . c + q_rot . k_rot) * scale, softmax, returns sum p c  [T, H, C]."""
+    T = q_abs.shape[0]
+    out = torch.zeros(T, H, C)
+    qa = q_abs.float().view(T, H, C)
+    qr = q.float().view(T, H, Dn + R)[..., Dn:]
+    for t in range(T):
+        p = int(positions[t])
+        if p < 0:
+            continue
+        lo = 0 if window <= 0 else max(0, p - window + 1)
+        js = torch.arange(lo, p + 1)
+        bt = block_tables[int(tok_seq[t])].long()
+        rows = cache[bt[js // block_size] * block_size + js % block_size].float()
+        s = (qa[t] @ rows[:, :C].T + qr[t] @ rows[:, C:].T) * scale
+        out[t] = torch.softmax(s, -1) @ rows[:, :C]
+    return out.to(out_dtype)
+
+
+# ----------------------------------------------------------------------------- mixture of experts
+def moe_route(logits: torch.Tensor, E: int, top: int, scale: float):
+    """softmax over the first E columns, the ``top`` largest (ties: lowest index), weights s / (sum s + 1e-20) * scale."""
+    s = torch.softmax(logits[:, :E].float(), -1)
+    w, idx = torch.sort(s, dim=-1, descending=True, stable=True)
+    w, idx = w[:, :top], idx[:, :top]
+    return idx.int().contiguous(), (w / (w.sum(-1, keepdim=True) + 1e-20) * scale).contiguous()
+
+
+def moe_align(topk_idx: torch.Tensor, E: int, BM: int):
+    """Sort the (token, choice) pairs by expert.  Returns sorted_tok [P] (token of each sorted row), pos_of_pair [P]
+    (sorted row of pair t * top + k), seg [E + 1] and the row tiles [(expert, row0, rows)] padded with expert -1."""
+    T, top = topk_idx.shape
+    flat = topk_idx.reshape(-1).long()
+    order = torch.sort(flat, stable=True).indices
+    pos = torch.empty_like(order)
+    pos[order] = torch.arange(order.numel())
+    cnt = torch.bincount(flat, minlength=E)
+    seg = torch.zeros(E + 1, dtype=torch.int32)
+    seg[1:] = cnt.cumsum(0)
+    ntiles = (T * top + BM - 1) // BM + E
+    tiles = torch.full((ntiles, 3), -1, dtype=torch.int32)
+    i = 0
+    for e in range(E):
+        for r0 in range(int(seg[e]), int(seg[e + 1]), BM):
+            tiles[i] = torch.tensor([e, r0, min(BM, int(seg[e + 1]) - r0)])
+            i += 1
+    return (order // top).int(), pos.int(), seg, tiles
+
+
+def moe_combine(D, pos_of_pair, topk_w, shared, logits, sg_col: int, out_dtype):
+    """z[t] = sum_k w[t, k] D[pos[t, k]] + sigmoid(logits[t, sg_col]) * shared[t]."""
+    T, top = topk_w.shape
+    z = (D.float()[pos_of_pair.long().view(T, top)] * topk_w.unsqueeze(-1)).sum(1)
+    if shared is not None:
+        gate = torch.sigmoid(logits[:, sg_col].float()).unsqueeze(-1) if sg_col >= 0 else 1.0
+        z = z + gate * shared.float()
+    return z.to(out_dtype)

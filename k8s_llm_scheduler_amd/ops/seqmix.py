@@ -1,0 +1,298 @@
+"""Ops of models with an fp32 residual stream, recurrent / latent-attention mixers and mixtures of experts.
+
+Same dispatch rule as the rest of :mod:`..ops`: CUDA (= HIP) tensors always run the gfx950 kernels
+(``stream32.hip``, ``mixers.hip``, ``moe.hip``) and raise when the extension is missing; CPU tensors run the fp32
+reference in :mod:`.reference` (the CPU test-suite).  Every op takes bf16 or true-fp32 activations / weights (the
+``f32`` flag of the kernels); what a design computes in fp32 regardless (residual sum, recurrent state, decays, router,
+attention scores) is fp32 in both.
+"""
+
+from __future__ import annotations
+
+import os
+from typing import Optional
+
+import torch
+
+from . import reference as ref
+from .reference import ACT_GELU_TANH, ACT_SILU, ACT_SWISH_CLAMP, ACT_TANH  # noqa: F401
+
+BF16, F32, I32 = torch.bfloat16, torch.float32, torch.int32
+GROUP_BM = 64   # row-tile height of the grouped GEMM (gemm_any_kernel's BM)
+
+
+def _native():
+    from . import native
+
+    return native()
+
+
+def _gpu(*ts) -> bool:
+    cuda = [t.is_cuda for t in ts if t is not None]
+    if any(cuda) and not all(cuda):
+        raise ValueError("mixed CPU/GPU tensors")
+    return bool(cuda) and cuda[0]
+
+
+def _p(t: Optional[torch.Tensor], dtype=None, name: str = "tensor") -> int:
+    if t is None:
+        return 0
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name}: expected {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: must be contiguous")
+    return t.data_ptr()
+
+
+def _f32(dtype) -> int:
+    if dtype == F32:
+        return 1
+    if dtype == BF16:
+        return 0
+    raise TypeError(f"activations must be bfloat16 or float32, got {dtype}")
+
+
+# ----------------------------------------------------------------------------- residual stream
+def embed_rows(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """fp32 [T, W] rows of ``table`` (bf16 or fp32)."""
+    if not _gpu(ids, table):
+        return ref.embed_rows(ids, table)
+    T, W = ids.shape[0], table.shape[1]
+    out = torch.empty(T, W, dtype=F32, device=table.device)
+    _native().embed_rows(out.data_ptr(), _p(ids, I32, "ids"), _p(table), T, W, table.shape[0], _f32(table.dtype), -1)
+    return out
+
+
+def resnorm(x: torch.Tensor, w: Optional[torch.Tensor], eps: float, *, branch: Optional[torch.Tensor] = None,
+            mult: float = 1.0, rowvec: Optional[torch.Tensor] = None, offset: float = 0.0,
+            out_dtype=BF16) -> Optional[torch.Tensor]:
+    """``x`` (fp32 [T, W], updated in place) += mult * branch + rowvec; returns rms-norm(x) * (offset + w) in
+    ``out_dtype``, or None when ``w`` is None (add only)."""
+    if x.dtype != F32:
+        raise TypeError("the residual stream is fp32")
+    if not _gpu(x, w, branch, rowvec):
+        return ref.resnorm(x, branch, mult, rowvec, w, offset, eps, out_dtype)
+    T, W = x.shape
+    out = torch.empty(T, W, dtype=out_dtype, device=x.device) if w is not None else None
+    f32 = _f32(out_dtype)
+    for t, n in ((branch, "branch"), (rowvec, "rowvec"), (w, "w")):
+        if t is not None and t.dtype != out_dtype:
+            raise TypeError(f"{n}: expected {out_dtype}, got {t.dtype}")
+    _native().resnorm(_p(x), _p(branch), float(mult), _p(rowvec), _p(w), float(offset), float(eps), _p(out), T, W,
+                      f32, -1)
+    return out
+
+
+def act(x: torch.Tensor, kind: int, limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
+    """Gated kinds (ACT_GELU_TANH, ACT_SWISH_CLAMP): [T, 2F] = [gate | up] -> [T, F]; ACT_TANH / ACT_SILU: elementwise."""
+    if not _gpu(x):
+        return ref.act(x, kind, limit, alpha)
+    T = x.shape[0]
+    F = x.shape[1] // 2 if kind in (ACT_GELU_TANH, ACT_SWISH_CLAMP) else x.shape[1]
+    out = torch.empty(T, F, dtype=x.dtype, device=x.device)
+    _native().act(out.data_ptr(), _p(x), T, F, kind, float(limit or 0.0), float(alpha), _f32(x.dtype), -1)
+    return out
+
+
+def _route_fast(a: torch.Tensor, w: torch.Tensor, out_dtype) -> bool:
+    """bf16 products whose shape the framework's tuned GEMV / MFMA GEMM kernels take (128-byte k steps, N % 4 == 0)."""
+    from . import GEMM_BACKEND
+
+    if a.dtype != BF16 or w.dtype != BF16 or out_dtype not in (BF16, F32) or a.dim() != 2 or w.dim() != 2:
+        return False
+    if GEMM_BACKEND == "library" or not a.is_contiguous() or not w.is_contiguous():
+        return False
+    N, K = w.shape
+    return K % 64 == 0 and N % 16 == 0 and K >= 128 and N >= 64
+
+
+# route fitting bf16 shapes to ops.linear (K8S_SEQMIX_FAST_GEMM=0: every product on the any-shape kernel)
+FAST_GEMM = os.environ.get("K8S_SEQMIX_FAST_GEMM", "1") != "0"
+
+
+def linear(a: torch.Tensor, w: torch.Tensor, out_dtype=None) -> torch.Tensor:
+    """a [M, K] @ w [N, K]^T for any shape, bf16 or fp32 operands (fp32: plain fp32 FMAs, no reduced-precision
+    matrix mode), fp32 accumulation.  Shapes that fit the tuned bf16 kernels go there."""
+    out_dtype = out_dtype or a.dtype
+    if not _gpu(a, w):
+        return ref.gemm_any(a, w, out_dtype)
+    if FAST_GEMM and _route_fast(a, w, out_dtype):
+        from . import linear as tuned
+
+        return tuned(a, w, out_dtype=F32 if out_dtype == F32 else None)
+    return gemm(a, w, out_dtype)
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, out_dtype=None, *, a_rows: Optional[torch.Tensor] = None,
+         tiles: Optional[torch.Tensor] = None, rows: Optional[int] = None,
+         seg: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The any-shape GEMM.  2-D: a [M, K] (row stride free) @ w [N, K]^T.  3-D: batched over dim 0 (a [G, M, K] with any
+    strides whose last is 1, w [G, N, K]) -> [G, M, N] (``out``: a [G, M, N] view with any batch / row strides).  Grouped (``tiles`` [n, 3] from :func:`moe_align`, w [G, N, K]):
+    ``rows`` compact rows, row r = a[a_rows[r]] (or a[r]), the rows of tile (g, r0, n) use w[g] -> [rows, N]."""
+    out_dtype = out_dtype or a.dtype
+    if a.dtype != w.dtype:
+        raise TypeError(f"gemm operands differ in dtype: {a.dtype} and {w.dtype}")
+    if a.stride(-1) != 1 or w.stride(-1) != 1:
+        raise ValueError("gemm: the k dimension must be contiguous")
+    if tiles is not None:
+        G, N, K = w.shape
+        if a.shape[-1] != K:
+            raise ValueError("gemm: k mismatch")
+        if not _gpu(a, w):
+            return ref.gemm_any(a, w, out_dtype, a_rows, tiles, seg)
+        out = torch.empty(rows, N, dtype=out_dtype, device=a.device)
+        _native().gemm_any(out.data_ptr(), a.data_ptr(), _p(w), rows, N, K, a.stride(0), K, N, 1, 0, N * K, 0,
+                           _p(a_rows, I32, "a_rows"), _p(tiles, I32, "tiles"), tiles.shape[0], _f32(a.dtype),
+                           _f32(out_dtype), -1)
+        return out
+    if a.shape[-1] != w.shape[-1]:
+        raise ValueError(f"gemm: k mismatch {tuple(a.shape)} x {tuple(w.shape)}")
+    if not _gpu(a, w):
+        y = ref.gemm_any(a, w, out_dtype)
+        if out is not None:
+            out.copy_(y)
+            return out
+        return y
+    if a.dim() == 2:
+        M, K = a.shape
+        N = w.shape[0]
+        out = torch.empty(M, N, dtype=out_dtype, device=a.device)
+        _native().gemm_any(out.data_ptr(), a.data_ptr(), w.data_ptr(), M, N, K, a.stride(0), w.stride(0), N, 1, 0, 0,
+                           0, 0, 0, 0, _f32(a.dtype), _f32(out_dtype), -1)
+        return out
+    G, M, K = a.shape
+    N = w.shape[1]
+    if out is None:
+        out = torch.empty(G, M, N, dtype=out_dtype, device=a.device)
+    elif out.shape != (G, M, N) or out.stride(2) != 1 or out.dtype != out_dtype:
+        raise ValueError("gemm: out must be a [G, M, N] view of the output dtype with contiguous rows")
+    _native().gemm_any(out.data_ptr(), a.data_ptr(), w.data_ptr(), M, N, K, a.stride(1), w.stride(1), out.stride(1), G,
+                       a.stride(0), w.stride(0), out.stride(0), 0, 0, 0, _f32(a.dtype), _f32(out_dtype), -1)
+    return out
+
+
+# ----------------------------------------------------------------------------- recurrent mixer
+def token_shift(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor, tok_seq: torch.Tensor,
+                seq_slots: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+    """[n, T, W]: h + (previous token's h - h) * mu[s]; the previous token of a portion's first token is the slot's
+    row of ``state`` (zeros at position 0)."""
+    if not _gpu(h, mu, state):
+        return ref.token_shift(h, mu, state, cu_q, seq_slots, positions)
+    T, W = h.shape
+    n = mu.shape[0]
+    out = torch.empty(n, T, W, dtype=h.dtype, device=h.device)
+    _native().token_shift(out.data_ptr(), _p(h), _p(mu, h.dtype, "mu"), _p(state, h.dtype, "state"),
+                          _p(cu_q, I32, "cu_q"), _p(tok_seq, I32, "tok_seq"), _p(seq_slots, I32, "seq_slots"),
+                          _p(positions, I32, "positions"), n, T, W, _f32(h.dtype), -1)
+    return out
+
+
+def shift_save(state: torch.Tensor, h: torch.Tensor, cu_q: torch.Tensor, seq_slots: torch.Tensor,
+               positions: torch.Tensor) -> None:
+    """state[slot of s] = h[last token of sequence s]."""
+    if not _gpu(h, state):
+        return ref.shift_save(state, h, cu_q, seq_slots, positions)
+    _native().shift_save(_p(state, h.dtype, "state"), _p(h), _p(cu_q, I32), _p(seq_slots, I32), _p(positions, I32),
+                         cu_q.shape[0] - 1, h.shape[1], _f32(h.dtype), -1)
+
+
+def wkv_max_dim() -> int:
+    return 128
+
+
+def wkv_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, z: torch.Tensor, w0: torch.Tensor,
+             u: torch.Tensor, lnw: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor, seq_slots: torch.Tensor,
+             positions: torch.Tensor, H: int, D: int, eps: float) -> torch.Tensor:
+    """The recurrence with its per-head unit norm, norm weight and silu gate; r, k, v, g [T, H D] (one row stride),
+    z [T, H D] fp32 decay logits (w = exp(-exp(z + w0))), ``state`` [slots, H, D, D] fp32 updated in place."""
+    T = r.shape[0]
+    if z.dtype != F32 or state.dtype != F32:
+        raise TypeError("decay logits and recurrent state are fp32")
+    if not _gpu(r, state):
+        return ref.wkv_scan(r, k, v, g, z, w0, u, lnw, state, cu_q, seq_slots, positions, H, D, eps, r.dtype)
+    if D > wkv_max_dim():
+        raise ValueError(f"wkv_scan: head dimension {D} exceeds the kernel's {wkv_max_dim()}")
+    ld = r.stride(0)
+    for t in (r, k, v, g):
+        if t.stride(0) != ld or t.stride(1) != 1 or t.dtype != r.dtype:
+            raise ValueError("wkv_scan: r, k, v, g must share dtype and row stride")
+    out = torch.empty(T, H * D, dtype=r.dtype, device=r.device)
+    _native().wkv_scan(out.data_ptr(), r.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), ld, _p(z),
+                       _p(w0, r.dtype, "w0"), _p(u, r.dtype, "u"), _p(lnw, r.dtype, "lnw"), _p(state),
+                       _p(cu_q, I32), _p(seq_slots, I32), _p(positions, I32), cu_q.shape[0] - 1, H, D, float(eps),
+                       _f32(r.dtype), -1)
+    return out
+
+
+# ----------------------------------------------------------------------------- latent attention
+def latent_kv_write(cache: torch.Tensor, dkv: torch.Tensor, normw: torch.Tensor, q: torch.Tensor,
+                    cos_sin: torch.Tensor, positions: torch.Tensor, slot_mapping: torch.Tensor, C: int, R: int, H: int,
+                    Dn: int, rot_dims: int, eps: float) -> None:
+    """cache[slot] = [rms-norm(dkv[:, :C]) * normw | rotated dkv[:, C:]]; rotates the last R of every head of q
+    ([T, H (Dn + R)]) in place.  ``cos_sin`` [positions, rot_dims] = [cos | sin] fp32."""
+    if not _gpu(cache, dkv, q):
+        return ref.latent_kv_write(cache, dkv, normw, q, cos_sin, positions, slot_mapping, C, R, H, Dn, rot_dims, eps)
+    dt = dkv.dtype
+    _native().latent_kv_write(_p(cache, dt, "cache"), _p(dkv), _p(normw, dt, "normw"), _p(q, dt, "q"),
+                              _p(cos_sin, F32, "cos_sin"), _p(positions, I32), _p(slot_mapping, I32), dkv.shape[0], C,
+                              R, H, Dn, rot_dims, float(eps), _f32(dt), -1)
+
+
+def latent_attention(q_abs: torch.Tensor, q: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor,
+                     tok_seq: torch.Tensor, positions: torch.Tensor, C: int, R: int, H: int, Dn: int, window: int,
+                     scale: float, block_size: int) -> torch.Tensor:
+    """Sliding-window attention in the latent space over the paged cache; returns softmax-weighted latents [T, H, C]."""
+    if not _gpu(q_abs, q, cache):
+        return ref.latent_attention(q_abs, q, cache, block_tables, tok_seq, positions, C, R, H, Dn, window, scale,
+                                    block_size, q.dtype)
+    T = q.shape[0]
+    dt = q.dtype
+    out = torch.empty(T, H, C, dtype=dt, device=q.device)
+    _native().latent_attention(out.data_ptr(), _p(q_abs, dt, "q_abs"), _p(q), _p(cache, dt, "cache"),
+                               _p(block_tables, I32, "block_tables"), block_tables.shape[1], _p(tok_seq, I32),
+                               _p(positions, I32), T, C, R, H, Dn, int(window), float(scale), block_size, _f32(dt), -1)
+    return out
+
+
+# ----------------------------------------------------------------------------- mixture of experts
+def moe_route(logits: torch.Tensor, E: int, top: int, scale: float):
+    """fp32 router logits [T, >= E] -> (expert ids int32 [T, top], weights fp32 [T, top])."""
+    if logits.dtype != F32:
+        raise TypeError("router logits are fp32")
+    if not _gpu(logits):
+        return ref.moe_route(logits, E, top, scale)
+    T = logits.shape[0]
+    idx = torch.empty(T, top, dtype=I32, device=logits.device)
+    w = torch.empty(T, top, dtype=F32, device=logits.device)
+    _native().moe_route(idx.data_ptr(), w.data_ptr(), _p(logits), logits.stride(0), T, E, top, float(scale), -1)
+    return idx, w
+
+
+def moe_align(topk_idx: torch.Tensor, E: int):
+    """(sorted_tok [P], pos_of_pair [P], seg [E + 1], tiles [n, 3]) for the grouped GEMMs; no host sync."""
+    if not _gpu(topk_idx):
+        return ref.moe_align(topk_idx, E, GROUP_BM)
+    T, top = topk_idx.shape
+    P = T * top
+    ntiles = (P + GROUP_BM - 1) // GROUP_BM + E
+    dev = topk_idx.device
+    sorted_tok = torch.empty(P, dtype=I32, device=dev)
+    pos = torch.empty(P, dtype=I32, device=dev)
+    seg = torch.empty(E + 1, dtype=I32, device=dev)
+    tiles = torch.empty(ntiles, 3, dtype=I32, device=dev)
+    _native().moe_align(sorted_tok.data_ptr(), pos.data_ptr(), seg.data_ptr(), tiles.data_ptr(), ntiles,
+                        _p(topk_idx, I32, "topk_idx"), P, top, E, GROUP_BM, -1)
+    return sorted_tok, pos, seg, tiles
+
+
+def moe_combine(D: torch.Tensor, pos_of_pair: torch.Tensor, topk_w: torch.Tensor, shared: Optional[torch.Tensor],
+                logits: torch.Tensor, sg_col: int) -> torch.Tensor:
+    """z[t] = sum_k w[t, k] D[pos[t, k]] + sigmoid(logits[t, sg_col]) * shared[t]  (sg_col < 0: ungated)."""
+    if not _gpu(D, topk_w, shared):
+        return ref.moe_combine(D, pos_of_pair, topk_w, shared, logits, sg_col, D.dtype)
+    T, top = topk_w.shape
+    W = D.shape[1]
+    z = torch.empty(T, W, dtype=D.dtype, device=D.device)
+    _native().moe_combine(z.data_ptr(), _p(D), _p(pos_of_pair, I32), _p(topk_w, F32), _p(shared, D.dtype, "shared"),
+                          _p(logits, F32), logits.stride(0), sg_col, T, W, top, _f32(D.dtype), -1)
+    return z
