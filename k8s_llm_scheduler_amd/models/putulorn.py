@@ -571,7 +571,7 @@ class PutulornModel:
             if L.mlp is not None:
                 h = sm.resnorm(x, L.n2, c.rms_eps, branch=y, mult=c.residual_mult, offset=1.0, out_dtype=dt)
                 y = self._mlp(L.mlp, h)
-            sm.resnorm(x, None, c.rms_eps, branch=y, mult=c.residual_mult)
+            sm.resnorm(x, None, c.rms_eps, branch=y, mult=c.residual_mult, out_dtype=dt)
             outs.append(x.clone())
         return outs
 
