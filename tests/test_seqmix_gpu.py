@@ -1,0 +1,168 @@
+"""Every kernel of ops.seqmix against the fp32 PyTorch reference of the same op (ops.reference), in bf16 and in true
+fp32, at sizes that are not multiples of the tiles and at sizes that take the vectorised / MFMA paths."""
+
+import pytest
+import torch
+
+from k8s_llm_scheduler_amd.ops import reference as ref
+from k8s_llm_scheduler_amd.ops import seqmix as sm
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+DTYPES = [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)]
+T = 37
+
+
+def close(a, b, tol):
+    a, b = a.float().cpu(), b.float().cpu()
+    assert (a - b).abs().max().item() <= tol * max(b.abs().max().item(), 1e-6)
+
+
+def batch():
+    """Four sequences (one empty, one resumed mid-sequence, one starting at 0) over T tokens."""
+    cu = torch.tensor([0, 9, 10, 10, T], dtype=torch.int32)
+    pos = torch.cat([torch.arange(0, 9), torch.tensor([5]), torch.arange(3, 30)]).int()
+    slots = torch.tensor([2, 0, 1, 3], dtype=torch.int32)
+    tok_seq = torch.searchsorted(cu[1:].contiguous(), torch.arange(T, dtype=torch.int32), right=True).int()
+    return cu, pos, slots, tok_seq
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+def test_stream_ops(dt, tol):
+    torch.manual_seed(0)
+    W = 200
+    ids = torch.randint(0, 50, (T,), dtype=torch.int32)
+    table = torch.randn(50, W).to(dt)
+    close(sm.embed_rows(ids.to(DEV), table.to(DEV)), sm.embed_rows(ids, table), 0)
+    x, br, rv, w = torch.randn(T, W), torch.randn(T, W).to(dt), torch.randn(W).to(dt), (torch.randn(W) * 0.1).to(dt)
+    xg, xc = x.to(DEV).clone(), x.clone()
+    og = sm.resnorm(xg, w.to(DEV), 1e-6, branch=br.to(DEV), mult=0.3, rowvec=rv.to(DEV), offset=1.0, out_dtype=dt)
+    oc = sm.resnorm(xc, w, 1e-6, branch=br, mult=0.3, rowvec=rv, offset=1.0, out_dtype=dt)
+    close(og, oc, tol)
+    close(xg, xc, 1e-6)
+    assert sm.resnorm(xg, None, 1e-6, branch=br.to(DEV), mult=2.0, out_dtype=dt) is None
+    sm.resnorm(xc, None, 1e-6, branch=br, mult=2.0, out_dtype=dt)
+    close(xg, xc, 1e-6)
+    for kind in (sm.ACT_GELU_TANH, sm.ACT_SWISH_CLAMP, sm.ACT_TANH, sm.ACT_SILU):
+        a = torch.randn(T, 140).to(dt) * 2
+        close(sm.act(a.to(DEV), kind, 1.0, 1.702), sm.act(a, kind, 1.0, 1.702), tol)
+    a = torch.randn(T, 140).to(dt) * 3
+    close(sm.act(a.to(DEV), sm.ACT_SWISH_CLAMP, 0.0, 1.702), sm.act(a, sm.ACT_SWISH_CLAMP, 0.0, 1.702), tol)
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(37, 200, 96), (1, 16, 256), (130, 70, 16), (64, 64, 64), (5, 640, 255), (3, 7, 5),
+                                   (200, 136, 72), (65, 129, 1032)])
+def test_gemm_shapes(dt, tol, M, N, K):
+    torch.manual_seed(1)
+    a, w = torch.randn(M, K).to(dt), (torch.randn(N, K) / K ** 0.5).to(dt)
+    for out in (dt, torch.float32):
+        close(sm.gemm(a.to(DEV), w.to(DEV), out), sm.gemm(a, w, out), tol)
+    if dt == torch.float32:      # true fp32: far below any reduced-precision matrix mode
+        exact = a.double() @ w.double().T
+        assert (sm.gemm(a.to(DEV), w.to(DEV)).cpu().double() - exact).abs().max() < 1e-5 * max(1.0, K ** 0.5)
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+@pytest.mark.parametrize("H,Dn,R,C", [(6, 40, 24, 72), (3, 7, 5, 9)])
+def test_gemm_batched_strided(dt, tol, H, Dn, R, C):
+    torch.manual_seed(2)
+    q, uk = torch.randn(T, H * (Dn + R)).to(dt), (torch.randn(H, C, Dn) / Dn ** 0.5).to(dt)
+
+    def run(q, uk):
+        out = torch.empty(T, H, C, dtype=dt, device=q.device)
+        sm.gemm(q.view(T, H, Dn + R)[:, :, :Dn].permute(1, 0, 2), uk, out=out.permute(1, 0, 2))
+        return out
+
+    close(run(q.to(DEV), uk.to(DEV)), run(q, uk), tol)
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+def test_token_shift_and_save(dt, tol):
+    torch.manual_seed(3)
+    W = 200
+    cu, pos, slots, tok_seq = batch()
+    h, mu, st = torch.randn(T, W).to(dt), torch.rand(5, W).to(dt), torch.randn(4, W).to(dt)
+    d = lambda *ts: (t.to(DEV) for t in ts)
+    close(sm.token_shift(*d(h, mu, st, cu, tok_seq, slots, pos)), sm.token_shift(h, mu, st, cu, tok_seq, slots, pos), tol)
+    sg, sc = st.to(DEV).clone(), st.clone()
+    sm.shift_save(sg, *d(h, cu, slots, pos))
+    sm.shift_save(sc, h, cu, slots, pos)
+    close(sg, sc, 0)
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+@pytest.mark.parametrize("H,D", [(3, 48), (2, 32), (2, 80), (5, 20), (1, 128)])
+def test_wkv_scan(dt, tol, H, D):
+    torch.manual_seed(4)
+    cu, pos, slots, _ = batch()
+    HD = H * D
+    r, k, v, g = (torch.randn(T, HD).to(dt) for _ in range(4))
+    z, w0 = torch.randn(T, HD), (torch.rand(HD) * 3 - 2).to(dt)
+    u, lnw = (torch.randn(HD) * 0.5).to(dt), (1 + 0.1 * torch.randn(HD)).to(dt)
+    S = torch.randn(4, H, D, D)
+    Sg, Sc = S.to(DEV).clone(), S.clone()
+    og = sm.wkv_scan(*(t.to(DEV) for t in (r, k, v, g, z, w0, u, lnw)), Sg, cu.to(DEV), slots.to(DEV), pos.to(DEV), H, D, 1e-6)
+    oc = sm.wkv_scan(r, k, v, g, z, w0, u, lnw, Sc, cu, slots, pos, H, D, 1e-6)
+    close(og, oc, tol * 3)
+    close(Sg, Sc, 1e-4)
+    assert torch.equal(Sg[1].cpu(), S[1])        # the empty sequence's slot is untouched
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+@pytest.mark.parametrize("H,Dn,R,C,dims,win", [(6, 40, 24, 72, 24, 7), (3, 16, 8, 130, 4, 0), (10, 32, 32, 64, 32, 100),
+                                               (2, 64, 64, 512, 64, 20)])
+def test_latent_attention(dt, tol, H, Dn, R, C, dims, win):
+    torch.manual_seed(5)
+    cu, pos, slots, tok_seq = batch()
+    bs, per = 16, 2
+    L = C + R
+    cache = torch.randn(4 * per * bs, L).to(dt)
+    bt = torch.randperm(4 * per).view(4, per).int()         # disjoint blocks per sequence
+    slot_map = torch.tensor([int(bt[tok_seq[t], pos[t] // bs]) * bs + int(pos[t]) % bs for t in range(T)],
+                            dtype=torch.int32)
+    slot_map[9] = -1                                          # a row whose cache write is dropped
+    dkv, nw = torch.randn(T, L).to(dt), (1 + 0.1 * torch.randn(C)).to(dt)
+    q = torch.randn(T, H * (Dn + R)).to(dt)
+    cs = ref.rope_table(dims, 64, 10000.0)
+    cg, qg, cc, qc = cache.to(DEV).clone(), q.to(DEV).clone(), cache.clone(), q.clone()
+    sm.latent_kv_write(cg, dkv.to(DEV), nw.to(DEV), qg, cs.to(DEV), pos.to(DEV), slot_map.to(DEV), C, R, H, Dn, dims, 1e-6)
+    sm.latent_kv_write(cc, dkv, nw, qc, cs, pos, slot_map, C, R, H, Dn, dims, 1e-6)
+    close(cg, cc, tol)
+    close(qg, qc, tol)
+    qabs = torch.randn(T, H, C).to(dt) * 0.3
+    og = sm.latent_attention(qabs.to(DEV), qc.to(DEV), cc.to(DEV), bt.to(DEV), tok_seq.to(DEV), pos.to(DEV), C, R, H, Dn,
+                             win, 0.2, bs)
+    oc = sm.latent_attention(qabs, qc, cc, bt, tok_seq, pos, C, R, H, Dn, win, 0.2, bs)
+    close(og, oc, tol)
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+@pytest.mark.parametrize("E,top,F,W", [(16, 2, 24, 200), (70, 3, 24, 40), (4, 4, 7, 33), (8, 2, 64, 128)])
+def test_moe(dt, tol, E, top, F, W):
+    torch.manual_seed(6)
+    lg = torch.randn(T, E + 1) * 2
+    ig, wg = sm.moe_route(lg.to(DEV), E, top, 2.5)
+    ic, wc = sm.moe_route(lg, E, top, 2.5)
+    assert torch.equal(ig.cpu(), ic)
+    close(wg, wc, 1e-5)
+    stg, pg, sgg, tg = sm.moe_align(ig, E)
+    stc, pc, sgc, tc = sm.moe_align(ic, E)
+    assert torch.equal(sgg.cpu(), sgc)
+    for e in range(E):                                       # the same tokens under every expert, in any order
+        a, b = int(sgc[e]), int(sgc[e + 1])
+        assert sorted(stg.cpu()[a:b].tolist()) == sorted(stc[a:b].tolist())
+    assert torch.equal(stg.cpu()[pg.cpu().long()], torch.arange(T).repeat_interleave(top).int())
+    live = tg.cpu()[tg.cpu()[:, 0] >= 0]
+    assert int(live[:, 2].sum()) == T * top
+    hh, wgu, wd = torch.randn(T, W).to(dt), (torch.randn(E, 2 * F, W) / W ** 0.5).to(dt), (torch.randn(E, W, F) / F ** 0.5).to(dt)
+    sh = torch.randn(T, W).to(dt)
+
+    def run(hh, wgu, wd, sh, st_, p_, seg_, t_, w_, lg_):
+        gu = sm.gemm(hh, wgu, a_rows=st_, tiles=t_, rows=T * top, seg=seg_)
+        D = sm.gemm(sm.act(gu, sm.ACT_SWISH_CLAMP, 1.0, 1.702), wd, tiles=t_, rows=T * top, seg=seg_)
+        return sm.moe_combine(D, p_, w_, sh, lg_, E), sm.moe_combine(D, p_, w_, None, lg_, -1)
+
+    for a, b in zip(run(hh.to(DEV), wgu.to(DEV), wd.to(DEV), sh.to(DEV), stg, pg, sgg, tg, wg, lg.to(DEV)),
+                    run(hh, wgu, wd, sh, stc, pc, sgc, tc, wc, lg)):
+        close(a, b, tol)
