@@ -74,9 +74,20 @@ def main() -> int:
     ap.add_argument("--top-p", type=float, default=1.0,
                     help="nucleus sampling (the reference sends no top_p: provider default 1.0); < 1 captures the "
                          "decode graphs with the top-p passes")
+    ap.add_argument("--model-bench", action="store_true",
+                    help="instead of the headline workload: prefill / decode tokens/s of the registered model designs "
+                         "(Putulorn dense, Putulorn with experts, Llama) at equal layer sizes, random weights")
+    ap.add_argument("--model-bench-widths", default="2048,4096", help="(--model-bench) model widths, comma-separated")
     ap.add_argument("--verbose", action="store_true", help="engine INFO logs (init, autotune, graph capture)")
     args = ap.parse_args()
     t_start = time.perf_counter()
+    if args.model_bench:
+        from k8s_llm_scheduler_amd.engine import modelbench
+
+        rows = modelbench.run(widths=tuple(int(w) for w in args.model_bench_widths.split(",")), progress=lambda r: print(json.dumps(r), file=sys.stderr, flush=True))
+        print(json.dumps({"metric": "model_bench", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic",
+                          "rows": rows}))
+        return 0
 
     if "WORLD_SIZE" not in os.environ and args.gpus > 1 and args.simulate_tp <= 1:
         # `python bench.py --gpus N` without a launcher: start the N rank processes ourselves (one per GPU) before

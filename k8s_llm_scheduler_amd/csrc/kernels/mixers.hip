@@ -161,7 +161,10 @@ __global__ void latent_attention_kernel(TA* __restrict__ out, const TA* __restri
   extern __shared__ float smem[];
   const int t = blockIdx.x;
   const int p = positions[t];
-  if (p < 0) return;
+  if (p < 0) {   // idle row: defined output, nothing read
+    for (int i = threadIdx.x; i < H * C; i += blockDim.x) stf(out, (size_t)t * H * C + i, 0.f);
+    return;
+  }
   const int L = C + R, LP = L + 1;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, nw = blockDim.x >> 6;
   float* tile = smem;                     // [KB][LP]
@@ -221,6 +224,197 @@ __global__ void latent_attention_kernel(TA* __restrict__ out, const TA* __restri
         if (d < C) stf(out, ((size_t)t * H + hd) * C + d, acc[i] / l);
       }
     }
+  }
+}
+
+// Latent attention on the matrix cores (bf16 cache, C % 16 == 0, every part a multiple of 8 elements).  All heads of a
+// token attend the same cached rows, so a token's (up to 16) heads are the 16 columns of one MFMA tile:
+//   S^T[key][head] = K Q^T      A = 16 cached rows (from the LDS tile), B = the heads' queries [q_abs | q_rot]
+//   O[head][d]    += P C        A = the 32 keys' probabilities (registers, keys in the order the S^T tile left them),
+//                               B = the tile's latent columns through the transposing LDS read
+// one wave per (token, group of 16 heads, key split), 32 keys per step, scores / softmax / sums in fp32.  With
+// splits > 1 (few tokens: decoding) every split writes (max, sum, unnormalised O) and latent_merge_kernel joins them.
+typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
+
+template <int NDB>
+__global__ __launch_bounds__(64) void latent_attention_mfma_kernel(
+    bf16_t* __restrict__ out, float* __restrict__ pacc, float* __restrict__ pml, const bf16_t* __restrict__ q_abs,
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache, const int* __restrict__ block_tables, int max_blocks,
+    const int* __restrict__ tok_seq, const int* __restrict__ positions, int C, int R, int H, int Dn, int window,
+    float scale, int bs, int nsplit) {
+  extern __shared__ __attribute__((aligned(16))) char smem_b[];
+  char* smem = smem_b;
+  const int t = blockIdx.x, hg = blockIdx.y, split = blockIdx.z;
+  const int lane = threadIdx.x, li = lane & 15, g = lane >> 4;
+  const int L = C + R, rowb = (L + 8) * 2, ndb = C / 16, HP = gridDim.y * 16;
+  const int p = positions[t];
+  if (p < 0) {
+    if (nsplit == 1)
+      for (int i = lane; i < 16 * C; i += 64) {
+        const int hd = hg * 16 + i / C;
+        if (hd < H) out[((size_t)t * H + hd) * C + i % C] = 0;
+      }
+    return;
+  }
+  char* qlds = smem;                 // [16][L + 8] bf16
+  char* klds = smem + 16 * rowb;     // [32][L + 8] bf16
+  const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  const int ntiles = (p + 1 - lo + 31) / 32;
+  const int tps = (ntiles + nsplit - 1) / nsplit;
+  const int t0 = split * tps, t1 = min(ntiles, t0 + tps);
+  const int* btr = block_tables + (size_t)tok_seq[t] * max_blocks;
+  const int cpr = L / 8;             // 16-byte chunks per row
+  const u32x4 zero = u32x4{0u, 0u, 0u, 0u};
+  for (int idx = lane; idx < 16 * cpr; idx += 64) {
+    const int r = idx / cpr, c = idx - r * cpr, hd = hg * 16 + r;
+    u32x4 v = zero;
+    if (hd < H)
+      v = 8 * c < C ? *reinterpret_cast<const u32x4*>(q_abs + ((size_t)t * H + hd) * C + 8 * c)
+                    : *reinterpret_cast<const u32x4*>(q + ((size_t)t * H + hd) * (Dn + R) + Dn + (8 * c - C));
+    *reinterpret_cast<u32x4*>(qlds + r * rowb + 16 * c) = v;
+  }
+  f32x4 o[NDB];
+#pragma unroll
+  for (int n = 0; n < NDB; ++n) o[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+  const int nkk = (L + 31) / 32;
+  const int qd = li >> 2, pd = li & 3;
+  for (int tile = t0; tile < t1; ++tile) {
+    const int j0 = lo + tile * 32;
+    __syncthreads();
+    for (int idx = lane; idx < 32 * cpr; idx += 64) {
+      const int r = idx / cpr, c = idx - r * cpr, key = j0 + r;
+      u32x4 v = zero;
+      if (key <= p) {
+        const size_t slot = (size_t)btr[key / bs] * bs + (key % bs);
+        v = *reinterpret_cast<const u32x4*>(cache + slot * L + 8 * c);
+      }
+      *reinterpret_cast<u32x4*>(klds + r * rowb + 16 * c) = v;
+    }
+    __syncthreads();
+    f32x4 sacc[2];
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+      f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int kk = 0; kk < nkk; ++kk) {
+        const int piece = 32 * kk + 8 * g;
+        bf16x8 ka, qb;
+        if (piece < L) {
+          ka = *reinterpret_cast<const bf16x8*>(klds + (16 * m + li) * rowb + 2 * piece);
+          qb = *reinterpret_cast<const bf16x8*>(qlds + li * rowb + 2 * piece);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) { ka[e] = (__bf16)0.f; qb[e] = (__bf16)0.f; }
+        }
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb, acc, 0, 0, 0);
+      }
+      sacc[m] = acc;   // S[key j0 + 16 m + 4 g + i][head li]
+    }
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = j0 + 16 * m + 4 * g + i;
+        const float v = key <= p ? sacc[m][i] * scale : -INFINITY;
+        sacc[m][i] = v;
+        tmax = fmaxf(tmax, v);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+    const float m_new = fmaxf(m_run, tmax);       // finite: key j0 is always visible
+    const float alpha = m_run == -INFINITY ? 0.f : expf(m_run - m_new);
+    float rsum = 0.f;
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pv = expf(sacc[m][i] - m_new);
+        sacc[m][i] = pv;
+        rsum += pv;
+      }
+    rsum += __shfl_xor(rsum, 16, WAVE);
+    rsum += __shfl_xor(rsum, 32, WAVE);
+    l_run = l_run * alpha + rsum;
+    m_run = m_new;
+    float a_i[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a_i[i] = __shfl(alpha, g * 4 + i, WAVE);
+    bf16x8 pa;       // slot j < 4: key 4 g + j; slot j >= 4: key 16 + 4 g + (j - 4)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      pa[j] = (__bf16)sacc[0][j];
+      pa[4 + j] = (__bf16)sacc[1][j];
+    }
+    const int r0 = 4 * g + qd, r1 = r0 + 16;
+#pragma unroll
+    for (int n = 0; n < NDB; ++n) {
+      if (n < ndb) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[n][i] *= a_i[i];
+        const int col = 16 * n + 4 * pd;
+        const bf16x4 v0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(klds + r0 * rowb + 2 * col));
+        const bf16x4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(klds + r1 * rowb + 2 * col));
+        bf16x8 vb;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { vb[j] = v0[j]; vb[4 + j] = v1[j]; }
+        o[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vb, o[n], 0, 0, 0);
+      }
+    }
+  }
+  // o[n][i] = O[head 4 g + i][d 16 n + li]; the head's (max, sum) live in the lanes with li == head
+  float l_i[4], m_i[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    l_i[i] = __shfl(l_run, g * 4 + i, WAVE);
+    m_i[i] = __shfl(m_run, g * 4 + i, WAVE);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int hd = hg * 16 + 4 * g + i;
+    if (hd >= H) continue;
+    if (nsplit == 1) {
+      const float inv = 1.f / l_i[i];
+#pragma unroll
+      for (int n = 0; n < NDB; ++n)
+        if (n < ndb) out[((size_t)t * H + hd) * C + 16 * n + li] = f2bf(o[n][i] * inv);
+    } else {
+      const size_t rec = ((size_t)t * HP + hg * 16 + 4 * g + i) * nsplit + split;
+#pragma unroll
+      for (int n = 0; n < NDB; ++n)
+        if (n < ndb) pacc[rec * C + 16 * n + li] = o[n][i];
+      if (li == 0) {
+        pml[rec * 2] = m_i[i];      // -inf and 0 for a split without tiles
+        pml[rec * 2 + 1] = l_i[i];
+      }
+    }
+  }
+}
+
+// out[t][head] = sum_s e^(m_s - M) O_s / sum_s e^(m_s - M) l_s over the key splits
+__global__ void latent_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ pacc,
+                                    const float* __restrict__ pml, const int* __restrict__ positions, int C, int H,
+                                    int HP, int nsplit) {
+  const int t = blockIdx.x, hd = blockIdx.y;
+  if (positions[t] < 0) {
+    for (int d = threadIdx.x; d < C; d += blockDim.x) out[((size_t)t * H + hd) * C + d] = 0;
+    return;
+  }
+  const size_t rec0 = ((size_t)t * HP + hd) * nsplit;
+  float M = -INFINITY;
+  for (int s = 0; s < nsplit; ++s) M = fmaxf(M, pml[(rec0 + s) * 2]);
+  float den = 0.f;
+  for (int s = 0; s < nsplit; ++s) {
+    const float ms = pml[(rec0 + s) * 2];
+    if (ms != -INFINITY) den += expf(ms - M) * pml[(rec0 + s) * 2 + 1];
+  }
+  for (int d = threadIdx.x; d < C; d += blockDim.x) {
+    float a = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+      const float ms = pml[(rec0 + s) * 2];
+      if (ms != -INFINITY) a += expf(ms - M) * pacc[(rec0 + s) * C + d];
+    }
+    out[((size_t)t * H + hd) * C + d] = f2bf(a / den);
   }
 }
 
@@ -321,5 +515,30 @@ extern "C" int k8s_latent_attention(void* out, const void* q_abs, const void* q,
   else K8S_LA_T(bf16_t);
 #undef K8S_LA_T
 #undef K8S_LA
+  return (int)hipGetLastError();
+}
+
+// Whether the MFMA kernel takes these sizes (else the caller uses k8s_latent_attention).
+extern "C" int k8s_latent_mfma_ok(int C, int R, int Dn) {
+  const int L = C + R;
+  return C % 16 == 0 && R % 8 == 0 && Dn % 8 == 0 && C <= 512 && 48 * (L + 8) * 2 <= 64 * 1024;
+}
+
+extern "C" int k8s_latent_attention_mfma(void* out, float* pacc, float* pml, const void* q_abs, const void* q,
+                                         const void* cache, const int* block_tables, int max_blocks,
+                                         const int* tok_seq, const int* positions, int T, int C, int R, int H, int Dn,
+                                         int window, float scale, int bs, int nsplit, hipStream_t s) {
+  if (T <= 0) return 0;
+  if (!k8s_latent_mfma_ok(C, R, Dn) || H <= 0 || bs <= 0 || nsplit < 1 || (nsplit > 1 && (!pacc || !pml))) return -1;
+  const int L = C + R, HG = (H + 15) / 16;
+  const size_t lds = (size_t)48 * (L + 8) * 2;
+  const dim3 grid(T, HG, nsplit);
+#define K8S_LM(NDB)   latent_attention_mfma_kernel<NDB><<<grid, 64, lds, s>>>((bf16_t*)out, pacc, pml, (const bf16_t*)q_abs,                                                           (const bf16_t*)q, (const bf16_t*)cache, block_tables,                                                           max_blocks, tok_seq, positions, C, R, H, Dn, window, scale,                                                           bs, nsplit)
+  if (C <= 128) K8S_LM(8);
+  else if (C <= 256) K8S_LM(16);
+  else K8S_LM(32);
+#undef K8S_LM
+  if (nsplit > 1)
+    latent_merge_kernel<<<dim3(T, H), 128, 0, s>>>((bf16_t*)out, pacc, pml, positions, C, H, HG * 16, nsplit);
   return (int)hipGetLastError();
 }

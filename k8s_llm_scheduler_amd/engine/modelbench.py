@@ -1,0 +1,81 @@
+"""Prefill and decode throughput of the registered model designs at equal layer sizes (``bench.py --model-bench``).
+
+For every size a Putulorn (dense feed-forwards), a Putulorn with experts and a Llama of the same width, depth,
+feed-forward size and vocabulary are built with random weights and driven through the same engine entry points:
+
+* prefill: one whole prompt of ``T`` tokens in one step (``LLMEngine.replay_step``, the varlen forward), tokens/s;
+* decode: ``B`` requests generated together (``LLMEngine.generate``: captured decode graphs), new tokens/s from the
+  engine's GPU-event decode time.
+"""
+
+from __future__ import annotations
+
+import time
+from typing import Dict, List
+
+SIZES = {
+    # width: (layer pairs, ff, wkv head dim, latent heads, expert ff, experts)
+    2048: (4, 8192, 64, 16, 2048, 8),
+    4096: (2, 14336, 64, 32, 3584, 8),
+}
+VOCAB = 32768
+
+
+def _register(width: int) -> Dict[str, str]:
+    from ..models import putulorn
+    from ..models.config import PRESETS, LlamaConfig
+
+    pairs, ff, wd, heads, eff, experts = SIZES[width]
+    names = {"putulorn-dense": f"putulorn-w{width}-dense", "putulorn-moe": f"putulorn-w{width}-moe",
+             "llama": f"llama-w{width}"}
+    kw = dict(heads=heads, wkv_dim=wd, dim=128, rot_dim=64, vdim=128, kv_rank=512, window=1024, ff=ff)
+    putulorn.PRESETS[names["putulorn-dense"]] = putulorn.preset(names["putulorn-dense"], width, VOCAB, pairs, **kw)
+    putulorn.PRESETS[names["putulorn-moe"]] = putulorn.preset(names["putulorn-moe"], width, VOCAB, pairs, experts=experts,
+                                                            top=2, expert_ff=eff, **kw)
+    PRESETS[names["llama"]] = LlamaConfig(names["llama"], 2 * pairs, width, width // 128, max(1, width // 512), 128, ff,
+                                          VOCAB, bos_id=VOCAB - 256, eos_ids=(VOCAB - 255,), max_position=8192)
+    return names
+
+
+def run(widths=(2048, 4096), prefill_tokens=(512, 2048), decode_batches=(1, 8, 32), context: int = 512,
+        new_tokens: int = 32, repeats: int = 3, progress=print) -> List[dict]:
+    import torch
+
+    from . import build_engine
+    from .sampling import SamplingParams
+
+    rows = []
+    for width in widths:
+        for kind, name in _register(width).items():
+            maxb = max(decode_batches)
+            mml = max(max(prefill_tokens), context + new_tokens + 16)
+            eng = build_engine(name, max_batch=maxb, block_size=16, num_blocks=maxb * (mml // 16 + 1),
+                               max_model_len=mml, prefix_caching=False, max_prefill_tokens=max(prefill_tokens))
+            row = {"model": kind, "width": width, "layers": eng.model.cfg.num_layers,
+                   "weight_gb": round(eng.model.weight_bytes() / 1e9, 2)}
+            g = torch.Generator().manual_seed(0)
+            for T in prefill_tokens:
+                toks = torch.randint(0, VOCAB - 512, (T,), generator=g).tolist()
+                best = 1e9
+                for i in range(repeats + 1):
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    eng.replay_step([("p", toks, [T - 1])], ["p"])
+                    torch.cuda.synchronize()
+                    if i:
+                        best = min(best, time.perf_counter() - t0)
+                row[f"prefill_tok_s@{T}"] = round(T / best)
+            sp = SamplingParams(max_tokens=new_tokens, temperature=0.0, ignore_eos=True, stop_on_json_close=False)
+            for B in decode_batches:
+                prompts = [torch.randint(0, VOCAB - 512, (context,), generator=g).tolist() for _ in range(B)]
+                best = 0.0
+                for i in range(2):
+                    eng.stats["decode_time"], eng.stats["decode_tokens"] = 0.0, 0
+                    eng.generate(prompts, sp)
+                    best = max(best, eng.stats["decode_tokens"] / max(eng.stats["decode_time"], 1e-9))
+                row[f"decode_tok_s@B{B}"] = round(best)
+            progress(row)
+            rows.append(row)
+            del eng
+            torch.cuda.empty_cache()
+    return rows

@@ -213,27 +213,29 @@ def tensor_shapes(cfg: PutulornConfig) -> Dict[str, tuple]:
     return t
 
 
-def random_tensors(cfg: PutulornConfig, seed: int = 0) -> Dict[str, torch.Tensor]:
+def random_tensors(cfg: PutulornConfig, seed: int = 0, device="cpu") -> Dict[str, torch.Tensor]:
     """Random bf16 weights of a configuration (benchmarks and tests): projections ~ N(0, 1 / fan_in), norm weights and
     token-shift mixes small, decay offsets spread so that the heads forget at different rates."""
-    g = torch.Generator().manual_seed(seed)
+    g = torch.Generator(device=device).manual_seed(seed)
     out: Dict[str, torch.Tensor] = {}
+    rand = lambda shape, generator: torch.rand(shape, generator=generator, device=device)
+    randn = lambda shape, generator: torch.randn(shape, generator=generator, device=device)
     for name, shape in tensor_shapes(cfg).items():
         leaf = name.rsplit(".", 1)[-1]
         if ".mu." in name:
-            t = torch.rand(shape, generator=g)
+            t = rand(shape, g)
         elif leaf in ("norm", "norm1", "norm2") and len(shape) == 1:
-            t = torch.randn(shape, generator=g) * 0.1 + (1.0 if name.endswith("dkv.norm") or ".mix.norm" in name else 0.0)
+            t = randn(shape, g) * 0.1 + (1.0 if name.endswith("dkv.norm") or ".mix.norm" in name else 0.0)
         elif leaf == "w0":
-            t = torch.rand(shape, generator=g) * 4.0 - 3.0
+            t = rand(shape, g) * 4.0 - 3.0
         elif leaf == "u":
-            t = torch.randn(shape, generator=g) * 0.5
+            t = randn(shape, g) * 0.5
         elif leaf == "step":
-            t = torch.randn(shape, generator=g) * 0.1
+            t = randn(shape, g) * 0.1
         elif leaf == "embed":
-            t = torch.randn(shape, generator=g)
+            t = randn(shape, g)
         else:
-            t = torch.randn(shape, generator=g) / math.sqrt(shape[-1])
+            t = randn(shape, g) / math.sqrt(shape[-1])
         out[name] = t.to(torch.bfloat16)
     return out
 
@@ -354,7 +356,7 @@ class PutulornModel:
         self.block_size = 16
         self._rope: Dict[tuple, torch.Tensor] = {}
         if tensors is None:
-            tensors = self._open(Path(weights)) if weights else random_tensors(cfg, seed)
+            tensors = self._open(Path(weights)) if weights else random_tensors(cfg, seed, self.device)
         get = tensors if callable(tensors) else tensors.__getitem__
         self._build(get)
         self.runs: List[_Run] = []
@@ -517,7 +519,7 @@ class PutulornModel:
         q_abs = torch.empty(T, H, C, dtype=self.dtype, device=h.device)
         sm.gemm(q.view(T, H, Dn + R)[:, :, :Dn].permute(1, 0, 2), w.uk_t, out=q_abs.permute(1, 0, 2))
         lat = sm.latent_attention(q_abs, q, cache, b["block_tables"], b["tok_seq"], b["positions"], C, R, H, Dn,
-                                  m.window, m.scale, self.block_size)     # [T, H, C]
+                                  m.window, m.scale, self.block_size, b.get("max_keys", 0))     # [T, H, C]
         a = torch.empty(T, H, V, dtype=self.dtype, device=h.device)
         sm.gemm(lat.permute(1, 0, 2), w.uv, out=a.permute(1, 0, 2))
         return sm.linear(a.view(T, H * V), w.o)
@@ -610,7 +612,8 @@ class PutulornModel:
         slots = torch.where(context_lens > 0, blk * bs + pos % bs, torch.full_like(blk, -1)).to(torch.int32)
         ar = torch.arange(B + 1, dtype=torch.int32, device=dev)
         b = {"positions": (context_lens - 1).to(torch.int32), "slot_mapping": slots.contiguous(), "cu_q": ar,
-             "tok_seq": ar[:B], "block_tables": block_tables.contiguous(), "seq_slots": ar[:B]}
+             "tok_seq": ar[:B], "block_tables": block_tables.contiguous(), "seq_slots": ar[:B],
+             "max_keys": int(max_context)}
         return self._forward(tokens, b, ar[:B].long())
 
     def warm(self) -> None:

@@ -238,19 +238,46 @@ def latent_kv_write(cache: torch.Tensor, dkv: torch.Tensor, normw: torch.Tensor,
                               R, H, Dn, rot_dims, float(eps), _f32(dt), -1)
 
 
+LATENT_MFMA = os.environ.get("K8S_LATENT_MFMA", "1") != "0"   # 0: always the plain-FMA attention kernel
+
+
+def latent_splits(T: int, H: int, max_keys: int) -> int:
+    """Key splits of the MFMA latent attention: one when the (token, 16-head group) grid fills the chip by itself
+    (prefill), else enough splits of at least one 32-key step each for about 256 workgroups (decoding)."""
+    groups = T * ((H + 15) // 16)
+    if groups >= 128:
+        return 1
+    return max(1, min(256 // groups, (max(1, max_keys) + 31) // 32, 32))
+
+
 def latent_attention(q_abs: torch.Tensor, q: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor,
                      tok_seq: torch.Tensor, positions: torch.Tensor, C: int, R: int, H: int, Dn: int, window: int,
-                     scale: float, block_size: int) -> torch.Tensor:
-    """Sliding-window attention in the latent space over the paged cache; returns softmax-weighted latents [T, H, C]."""
+                     scale: float, block_size: int, max_keys: int = 0) -> torch.Tensor:
+    """Sliding-window attention in the latent space over the paged cache; returns softmax-weighted latents [T, H, C].
+    ``max_keys``: an upper bound of the keys any token sees (sizes the key splits; 0: the table's capacity).
+    bf16 with 16-byte-aligned parts runs on the matrix cores; fp32 and other sizes on the plain-FMA kernel."""
     if not _gpu(q_abs, q, cache):
         return ref.latent_attention(q_abs, q, cache, block_tables, tok_seq, positions, C, R, H, Dn, window, scale,
                                     block_size, q.dtype)
     T = q.shape[0]
     dt = q.dtype
     out = torch.empty(T, H, C, dtype=dt, device=q.device)
-    _native().latent_attention(out.data_ptr(), _p(q_abs, dt, "q_abs"), _p(q), _p(cache, dt, "cache"),
-                               _p(block_tables, I32, "block_tables"), block_tables.shape[1], _p(tok_seq, I32),
-                               _p(positions, I32), T, C, R, H, Dn, int(window), float(scale), block_size, _f32(dt), -1)
+    nat = _native()
+    args = (_p(q_abs, dt, "q_abs"), _p(q), _p(cache, dt, "cache"), _p(block_tables, I32, "block_tables"),
+            block_tables.shape[1], _p(tok_seq, I32), _p(positions, I32), T, C, R, H, Dn, int(window), float(scale),
+            block_size)
+    if LATENT_MFMA and dt == BF16 and nat.latent_mfma_ok(C, R, Dn):
+        cap = block_tables.shape[1] * block_size
+        bound = min(max_keys or cap, window or cap, cap)
+        ns = latent_splits(T, H, bound)
+        pacc = pml = None
+        if ns > 1:
+            HP = (H + 15) // 16 * 16
+            pacc = torch.empty(T * HP * ns * C, dtype=F32, device=q.device)
+            pml = torch.empty(T * HP * ns * 2, dtype=F32, device=q.device)
+        nat.latent_attention_mfma(out.data_ptr(), _p(pacc), _p(pml), *args, ns, -1)
+    else:
+        nat.latent_attention(out.data_ptr(), *args, _f32(dt), -1)
     return out
 
 

@@ -330,6 +330,21 @@ def test_other_sizes(tmp_path, device, case):
     assert rel_err(torch.cat(rows), want) < TOL["float32"]
 
 
+@pytest.mark.parametrize("device", DEVICES)
+def test_bfloat16_aligned_sizes_long_context(tmp_path, device):
+    """Sizes whose rows are 16-byte aligned (on the GPU: the matrix-core attention and GEMM kernels) in bfloat16:
+    a prompt in portions, then 70 tokens one by one across 32-key steps, with and without a window."""
+    cfg = config([with_mlp(latent(heads=4, dim=16, rot_dim=16, vdim=16, kv_rank=32, window=0, scale=0.18), dense(64)),
+                  with_mlp(wkv(heads=2, dim=32), moe(experts=4, top=2, ff=16)),
+                  latent(heads=20, dim=8, rot_dim=8, vdim=8, kv_rank=48, window=37, scale=0.25)], width=64, vocab=80)
+    eng, tensors = make(tmp_path, cfg, device, "bfloat16", max_tokens=256)
+    toks = tokens(190, 80, 12)
+    want = oracle.forward(cfg, tensors, toks)
+    rows = [eng.replay_step([("m", toks[:90], list(range(90)))]), eng.replay_step([("m", toks[90:120], list(range(30)))])]
+    rows += [eng.replay_step([("m", [t], [0])]) for t in toks[120:]]
+    assert close(torch.cat(rows), want, "bfloat16")
+
+
 # ----------------------------------------------------------------------------- generation entry point
 @pytest.mark.parametrize("device", DEVICES)
 def test_greedy_generation_through_the_scheduler(tmp_path, device):

@@ -111,7 +111,8 @@ def test_wkv_scan(dt, tol, H, D):
 
 @pytest.mark.parametrize("dt,tol", DTYPES)
 @pytest.mark.parametrize("H,Dn,R,C,dims,win", [(6, 40, 24, 72, 24, 7), (3, 16, 8, 130, 4, 0), (10, 32, 32, 64, 32, 100),
-                                               (2, 64, 64, 512, 64, 20)])
+                                               (2, 64, 64, 512, 64, 20), (20, 16, 8, 48, 8, 0), (16, 8, 24, 96, 24, 13),
+                                               (5, 32, 40, 272, 40, 33)])
 def test_latent_attention(dt, tol, H, Dn, R, C, dims, win):
     torch.manual_seed(5)
     cu, pos, slots, tok_seq = batch()
@@ -166,3 +167,27 @@ def test_moe(dt, tol, E, top, F, W):
     for a, b in zip(run(hh.to(DEV), wgu.to(DEV), wd.to(DEV), sh.to(DEV), stg, pg, sgg, tg, wg, lg.to(DEV)),
                     run(hh, wgu, wd, sh, stc, pc, sgc, tc, wc, lg)):
         close(a, b, tol)
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+@pytest.mark.parametrize("H,win", [(4, 0), (20, 0), (6, 40), (3, 64), (3, 65), (16, 1)])
+def test_latent_attention_long_contexts(dt, tol, H, win):
+    """Few tokens over long contexts: several 32-key steps, key splits and their merge, window starts that are not
+    multiples of the step, an idle row."""
+    torch.manual_seed(7)
+    C, R, Dn, bs, nb = 96, 32, 24, 16, 20
+    pos = torch.tensor([299, 300, 31, 32, 33, -1, 64, 130], dtype=torch.int32)
+    tok_seq = torch.tensor([0, 0, 1, 1, 1, 2, 3, 3], dtype=torch.int32)
+    Tn = pos.numel()
+    bt = torch.randperm(4 * nb).view(4, nb).int()
+    cache = torch.randn(4 * nb * bs, C + R).to(dt)
+    q = torch.randn(Tn, H * (Dn + R)).to(dt)
+    qabs = (torch.randn(Tn, H, C) * 0.3).to(dt)
+    for max_keys in (0, 512):
+        og = sm.latent_attention(qabs.to(DEV), q.to(DEV), cache.to(DEV), bt.to(DEV), tok_seq.to(DEV), pos.to(DEV), C, R, H,
+                                 Dn, win, 0.15, bs, max_keys)
+        oc = sm.latent_attention(qabs, q, cache, bt, tok_seq, pos, C, R, H, Dn, win, 0.15, bs)
+        live = pos >= 0
+        close(og.cpu()[live], oc[live], tol)
+        assert torch.equal(og.cpu()[~live].float(), torch.zeros(1, H, C))
+    assert sm.latent_splits(Tn, H, 512) > 1 and sm.latent_splits(4096, H, 512) == 1
