@@ -122,9 +122,11 @@ int k8s_token_shift(void* out, const void* h, const void* mu, const void* state,
 int k8s_shift_save(void* state, const void* h, const int* cu_q, const int* seq_slots, const int* positions, int nseq,
                    int W, int f32, hipStream_t s);
 int k8s_wkv_max_dim();
+long long k8s_wkv_workspace(int T, int nseq, int H, int D, int Lc);
 int k8s_wkv_scan(void* out, const void* r, const void* k, const void* v, const void* g, long ld, const float* z,
                  const void* w0, const void* u, const void* lnw, float* state, const int* cu_q, const int* seq_slots,
-                 const int* positions, int nseq, int H, int D, float eps, int f32, hipStream_t s);
+                 const int* positions, int nseq, int H, int D, float eps, int f32, int T, int Lc, float* ws,
+                 hipStream_t s);
 int k8s_latent_kv_write(void* cache, const void* dkv, const void* normw, void* q, const float* cos_sin,
                         const int* positions, const int* slot_mapping, int T, int C, int R, int H, int Dn, int dims,
                         float eps, int f32, hipStream_t s);
@@ -410,10 +412,13 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
   m.def("wkv_max_dim", []() { return k8s_wkv_max_dim(); });
   m.def("wkv_scan", [](uintptr_t out, uintptr_t r, uintptr_t k, uintptr_t v, uintptr_t g, long ld, uintptr_t z,
                        uintptr_t w0, uintptr_t u, uintptr_t lnw, uintptr_t state, uintptr_t cu_q, uintptr_t seq_slots,
-                       uintptr_t positions, int nseq, int H, int D, float eps, int f32, int64_t s) {
+                       uintptr_t positions, int nseq, int H, int D, float eps, int f32, int T, int Lc, uintptr_t ws,
+                       int64_t s) {
     check(k8s_wkv_scan(P(out), P(r), P(k), P(v), P(g), ld, P<float>(z), P(w0), P(u), P(lnw), P<float>(state),
-                       P<int>(cu_q), P<int>(seq_slots), P<int>(positions), nseq, H, D, eps, f32, S(s)), "wkv_scan");
+                       P<int>(cu_q), P<int>(seq_slots), P<int>(positions), nseq, H, D, eps, f32, T, Lc, P<float>(ws),
+                       S(s)), "wkv_scan");
   });
+  m.def("wkv_workspace", [](int T, int nseq, int H, int D, int Lc) { return k8s_wkv_workspace(T, nseq, H, D, Lc); });
   m.def("latent_kv_write", [](uintptr_t cache, uintptr_t dkv, uintptr_t normw, uintptr_t q, uintptr_t cos_sin,
                               uintptr_t positions, uintptr_t slots, int T, int C, int R, int H, int Dn, int dims,
                               float eps, int f32, int64_t s) {

@@ -41,65 +41,202 @@ __global__ void shift_save_kernel(TA* __restrict__ state, const TA* __restrict__
   for (int i = threadIdx.x; i < W; i += blockDim.x) state[dst + i] = h[src + i];
 }
 
-// One workgroup per (sequence, head), thread j owns column j of the head's state S[i][j] (i: key channel, j: value
-// channel) in registers.  Per token:  o_j = sum_i r_i (S_ij + u_i k_i v_j);  S_ij = w_i S_ij + k_i v_j  with
-// w = exp(-exp(z + w0)) in fp32; then the head's o / rms(o) * lnw * silu(g).
-template <typename TA, int DMAX>
-__global__ void wkv_scan_kernel(TA* __restrict__ out, const TA* __restrict__ r, const TA* __restrict__ k,
-                                const TA* __restrict__ v, const TA* __restrict__ g, long ld,
-                                const float* __restrict__ z, const TA* __restrict__ w0, const TA* __restrict__ u,
-                                const TA* __restrict__ lnw, float* __restrict__ state, const int* __restrict__ cu_q,
-                                const int* __restrict__ seq_slots, const int* __restrict__ positions, int H, int D,
-                                float eps) {
-  __shared__ float sr[DMAX], sk[DMAX], sw[DMAX], su[DMAX], red[16];
-  const int s = blockIdx.x, hd = blockIdx.y;
-  const int a = cu_q[s], b = cu_q[s + 1];
-  if (b <= a) return;
-  const int p0 = positions[a];
-  if (p0 < 0) return;
-  const int j = threadIdx.x;
+// Workgroup barrier that waits for this wave's LDS traffic only: __syncthreads() also drains the outstanding global
+// loads, which would put the prefetched inputs of the next tokens back on the recurrence's latency chain.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0); vmcnt and expcnt untouched
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+// Chunk g of a varlen batch cut into chunks of Lc tokens per sequence: (sequence, chunk in the sequence, chunks of the
+// sequence), or sequence -1 when g is past the last chunk.  Idle (position < 0) and empty sequences have no chunks.
+struct WkvChunk { int s, c, n; };
+__device__ __forceinline__ WkvChunk wkv_find_chunk(int g, const int* cu_q, const int* positions, int nseq, int Lc) {
+  for (int s = 0; s < nseq; ++s) {
+    const int a = cu_q[s], len = cu_q[s + 1] - a;
+    const int n = (len > 0 && positions[a] >= 0) ? (len + Lc - 1) / Lc : 0;
+    if (g < n) return WkvChunk{s, g, n};
+    g -= n;
+  }
+  return WkvChunk{-1, 0, 0};
+}
+
+// One workgroup per (sequence or chunk, head).  The head's state S[i][j] (i: key channel, j: value channel) lives in
+// registers: thread (j, c) owns column j of the CH key channels [c CH, (c + 1) CH), so the per-token chain of a wave is
+// CH steps, not D.  Per token:  o_j = sum_i r_i (S_ij + u_i k_i v_j);  S_ij = w_i S_ij + k_i v_j  with
+// w = exp(-exp(z + w0)) in fp32; the channel groups' partial o_j meet in LDS, then group 0 applies the head's
+// o / rms(o) * lnw * silu(g).  The next token's inputs are loaded while the current one is computed, and the barriers
+// wait for LDS traffic only.  blockDim = (DV, NS): DV = D rounded up to 64, NS = ceil(D / CH).
+//
+// MODE 0: a whole sequence per workgroup, from the slot's state (zero at position 0) to the slot's state.
+// Long prompts run as three passes over chunks of Lc tokens, so the recurrence is parallel over chunks:
+// MODE 1: a chunk from a zero state, no outputs: its state contribution and the product of its decays -> cs_loc, cs_dec;
+//         wkv_prefix_kernel then walks a sequence's chunks: start[c + 1] = dec[c] * start[c] + loc[c];
+// MODE 2: a chunk from its start state with outputs; a sequence's last chunk leaves the slot's state.
+template <typename TA, int CH, int MODE>
+__global__ __launch_bounds__(1024) void wkv_scan_kernel(TA* __restrict__ out, const TA* __restrict__ r,
+                                                        const TA* __restrict__ k, const TA* __restrict__ v,
+                                                        const TA* __restrict__ g, long ld, const float* __restrict__ z,
+                                                        const TA* __restrict__ w0, const TA* __restrict__ u,
+                                                        const TA* __restrict__ lnw, float* __restrict__ state,
+                                                        const int* __restrict__ cu_q, const int* __restrict__ seq_slots,
+                                                        const int* __restrict__ positions, int H, int D, float eps,
+                                                        int nseq, int Lc, float* __restrict__ cs_loc,
+                                                        float* __restrict__ cs_dec, const float* __restrict__ cs_start) {
+  constexpr int DMAX = 128;
+  __shared__ __attribute__((aligned(16))) float sr[DMAX], sk[DMAX], sw[DMAX], su[DMAX];
+  __shared__ float po[DMAX / CH][DMAX];
+  __shared__ float red[4];
+  const int hd = blockIdx.y;
+  int s, a, b, p0;
+  bool from_zero, last = true;
+  if (MODE == 0) {
+    s = blockIdx.x;
+    a = cu_q[s];
+    b = cu_q[s + 1];
+    if (b <= a) return;
+    p0 = positions[a];
+    if (p0 < 0) return;
+    from_zero = p0 == 0;
+  } else {
+    const WkvChunk ck = wkv_find_chunk(blockIdx.x, cu_q, positions, nseq, Lc);
+    if (ck.s < 0) return;
+    s = ck.s;
+    last = ck.c == ck.n - 1;
+    if (MODE == 1 && last) return;          // nothing follows a sequence's last chunk
+    a = cu_q[s] + ck.c * Lc;
+    b = min(cu_q[s + 1], a + Lc);
+    p0 = positions[a];
+    from_zero = MODE == 1 || p0 == 0;
+  }
+  const int j = threadIdx.x, c = threadIdx.y, NS = blockDim.y, DV = blockDim.x;
   const bool on = j < D;
-  const int HD = H * D;
+  const int HD = H * D, i0 = c * CH;
   float* st = state + ((size_t)seq_slots[s] * H + hd) * D * D;
-  float S[DMAX];
+  const size_t crec = ((size_t)blockIdx.x * H + hd) * D * D;     // this chunk's record in cs_loc / cs_start
+  const float* src = (MODE == 2 && a != cu_q[s]) ? cs_start + crec : st;
+  float S[CH], decp[CH];
 #pragma unroll
-  for (int i = 0; i < DMAX; ++i) S[i] = (on && i < D && p0 > 0) ? st[(size_t)i * D + j] : 0.f;
+  for (int e = 0; e < CH; ++e) {
+    S[e] = (on && i0 + e < D && !from_zero) ? src[(size_t)(i0 + e) * D + j] : 0.f;
+    decp[e] = 1.f;
+  }
   float w0j = 0.f, lnj = 0.f;
-  if (on) {
+  if (c == 0) {                       // group 0 stages the token's r, k, w (and u once); channels >= D stay zero
+    for (int x = j; x < DMAX; x += DV) sr[x] = sk[x] = sw[x] = su[x] = 0.f;
+  }
+  lds_barrier();
+  if (c == 0 && on) {
     su[j] = ldf(u, (size_t)hd * D + j);
     w0j = ldf(w0, (size_t)hd * D + j);
     lnj = ldf(lnw, (size_t)hd * D + j);
   }
-  for (int t = a; t < b; ++t) {
-    const size_t base = (size_t)t * ld + (size_t)hd * D + j;
-    float vj = 0.f, gj = 0.f;
-    if (on) {
-      sr[j] = ldf(r, base);
-      sk[j] = ldf(k, base);
-      sw[j] = expf(-expf(z[(size_t)t * HD + (size_t)hd * D + j] + w0j));
-      vj = ldf(v, base);
-      gj = ldf(g, base);
-    }
-    __syncthreads();
-    float o = 0.f;
-#pragma unroll
-    for (int i = 0; i < DMAX; ++i) {
-      if (i < D) {
-        const float kv = sk[i] * vj;
-        o = fmaf(sr[i], fmaf(su[i], kv, S[i]), o);
-        S[i] = fmaf(sw[i], S[i], kv);
+  // inputs of the next token (group 0: r, k, z, g and v; the others: v only)
+  float nr = 0.f, nk = 0.f, nv = 0.f, ng = 0.f, nz = 0.f;
+  auto fetch = [&](int t) {
+    if (on && t < b) {
+      const size_t base = (size_t)t * ld + (size_t)hd * D + j;
+      nv = ldf(v, base);
+      if (c == 0) {
+        if (MODE != 1) {
+          nr = ldf(r, base);
+          ng = ldf(g, base);
+        }
+        nk = ldf(k, base);
+        nz = z[(size_t)t * HD + (size_t)hd * D + j];
       }
     }
-    const float ss = block_sum(on ? o * o : 0.f, red);   // (its barriers also order the next token's LDS writes)
-    if (on) {
-      const float y = o / sqrtf(ss / (float)D + eps) * lnj * (gj / (1.f + expf(-gj)));
+  };
+  fetch(a);
+  for (int t = a; t < b; ++t) {
+    const float cr = nr, ck = nk, cv = nv, cg = ng, cz = nz;
+    fetch(t + 1);
+    if (c == 0 && on) {
+      sr[j] = cr;
+      sk[j] = ck;
+      sw[j] = expf(-expf(cz + w0j));
+    }
+    lds_barrier();
+    float o4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int e0 = 0; e0 < CH; e0 += 4) {
+      const f32x4 r4 = *reinterpret_cast<const f32x4*>(&sr[i0 + e0]);
+      const f32x4 k4 = *reinterpret_cast<const f32x4*>(&sk[i0 + e0]);
+      const f32x4 w4 = *reinterpret_cast<const f32x4*>(&sw[i0 + e0]);
+      const f32x4 u4 = *reinterpret_cast<const f32x4*>(&su[i0 + e0]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float kv = k4[e] * cv;
+        if (MODE != 1) o4[e] = fmaf(r4[e], fmaf(u4[e], kv, S[e0 + e]), o4[e]);
+        S[e0 + e] = fmaf(w4[e], S[e0 + e], kv);
+        if (MODE == 1) decp[e0 + e] *= w4[e];
+      }
+    }
+    if (MODE == 1) {
+      lds_barrier();                   // the LDS rows are free for the next token
+      continue;
+    }
+    if (on) po[c][j] = (o4[0] + o4[1]) + (o4[2] + o4[3]);
+    lds_barrier();
+    float o = 0.f, ss = 0.f;
+    if (c == 0) {
+      if (on)
+        for (int x = 0; x < NS; ++x) o += po[x][j];
+      ss = wave_sum(on ? o * o : 0.f);
+      if (DV > 64 && (j & 63) == 0) red[j >> 6] = ss;
+    }
+    if (DV > 64) {                     // the head's value channels span two waves: one more exchange (uniform branch)
+      lds_barrier();
+      ss = red[0] + red[1];
+    }
+    if (c == 0 && on) {
+      const float y = o / sqrtf(ss / (float)D + eps) * lnj * (cg / (1.f + expf(-cg)));
       stf(out, (size_t)t * HD + (size_t)hd * D + j, y);
     }
   }
   if (on) {
+    float* dst = MODE == 1 ? cs_loc + crec : st;
+    if (MODE != 2 || last) {
 #pragma unroll
-    for (int i = 0; i < DMAX; ++i)
-      if (i < D) st[(size_t)i * D + j] = S[i];
+      for (int e = 0; e < CH; ++e)
+        if (i0 + e < D) dst[(size_t)(i0 + e) * D + j] = S[e];
+    }
+    if (MODE == 1 && j == 0) {
+#pragma unroll
+      for (int e = 0; e < CH; ++e)
+        if (i0 + e < D) cs_dec[((size_t)blockIdx.x * H + hd) * D + i0 + e] = decp[e];
+    }
+  }
+}
+
+// start[first chunk + c + 1] = dec[c] * start[c] + loc[c] along a sequence's chunks; start of chunk 0 is the slot's state
+// (or zero at position 0) and is read by the MODE 2 pass directly.  One workgroup per (sequence, head).
+__global__ void wkv_prefix_kernel(float* __restrict__ cs_start, const float* __restrict__ cs_loc,
+                                  const float* __restrict__ cs_dec, const float* __restrict__ state,
+                                  const int* __restrict__ cu_q, const int* __restrict__ seq_slots,
+                                  const int* __restrict__ positions, int H, int D, int Lc) {
+  const int s = blockIdx.x, hd = blockIdx.y;
+  int first = 0;
+  for (int x = 0; x < s; ++x) {
+    const int a = cu_q[x], len = cu_q[x + 1] - a;
+    first += (len > 0 && positions[a] >= 0) ? (len + Lc - 1) / Lc : 0;
+  }
+  const int a = cu_q[s], len = cu_q[s + 1] - a;
+  if (len <= 0 || positions[a] < 0) return;
+  const int n = (len + Lc - 1) / Lc;
+  if (n < 2) return;
+  const bool zero = positions[a] == 0;
+  const float* st = state + ((size_t)seq_slots[s] * H + hd) * D * D;
+  for (int e = threadIdx.x; e < D * D; e += blockDim.x) {
+    const int i = e / D;
+    float S = zero ? 0.f : st[e];
+    for (int c = 0; c + 1 < n; ++c) {
+      const size_t rec = (size_t)(first + c) * H + hd;
+      S = fmaf(cs_dec[rec * D + i], S, cs_loc[rec * D * D + e]);
+      cs_start[(rec + H) * D * D + e] = S;      // chunk first + c + 1
+    }
   }
 }
 
@@ -446,27 +583,41 @@ extern "C" int k8s_shift_save(void* state, const void* h, const int* cu_q, const
 
 extern "C" int k8s_wkv_max_dim() { return 128; }
 
+// ws (MODE 1 / 2 passes): floats for 2 x chunks x H x D x D states + chunks x H x D decay products, chunks =
+// ceil(T / Lc) + nseq; Lc == 0 (or no workspace): one workgroup per sequence.
+extern "C" long long k8s_wkv_workspace(int T, int nseq, int H, int D, int Lc) {
+  if (Lc <= 0) return 0;
+  const long long chunks = (T + Lc - 1) / Lc + nseq;
+  return chunks * H * ((long long)2 * D * D + D);
+}
+
 extern "C" int k8s_wkv_scan(void* out, const void* r, const void* k, const void* v, const void* g, long ld,
                             const float* z, const void* w0, const void* u, const void* lnw, float* state,
                             const int* cu_q, const int* seq_slots, const int* positions, int nseq, int H, int D,
-                            float eps, int f32, hipStream_t s) {
+                            float eps, int f32, int T, int Lc, float* ws, hipStream_t s) {
   if (nseq <= 0) return 0;
   if (H <= 0 || D <= 0 || D > 128 || H > 65535) return -1;
-  const dim3 grid(nseq, H);
-  const int threads = (D + 63) / 64 * 64;
-#define K8S_WKV(TA, DM) \
-  wkv_scan_kernel<TA, DM><<<grid, threads, 0, s>>>((TA*)out, (const TA*)r, (const TA*)k, (const TA*)v, (const TA*)g, \
-                                                   ld, z, (const TA*)w0, (const TA*)u, (const TA*)lnw, state, cu_q, \
-                                                   seq_slots, positions, H, D, eps)
-  if (f32) {
-    if (D <= 32) K8S_WKV(float, 32);
-    else if (D <= 64) K8S_WKV(float, 64);
-    else K8S_WKV(float, 128);
-  } else {
-    if (D <= 32) K8S_WKV(bf16_t, 32);
-    else if (D <= 64) K8S_WKV(bf16_t, 64);
-    else K8S_WKV(bf16_t, 128);
+  constexpr int CH = 16;
+  const dim3 block((D + 63) / 64 * 64, (D + CH - 1) / CH);
+#define K8S_WKV(TA, MODE, GX, LOC, DEC, START)                                                                        \
+  wkv_scan_kernel<TA, CH, MODE><<<dim3(GX, H), block, 0, s>>>((TA*)out, (const TA*)r, (const TA*)k, (const TA*)v,      \
+                                                              (const TA*)g, ld, z, (const TA*)w0, (const TA*)u,        \
+                                                              (const TA*)lnw, state, cu_q, seq_slots, positions, H, D, \
+                                                              eps, nseq, Lc, LOC, DEC, START)
+  if (Lc <= 0 || ws == nullptr) {
+    if (f32) K8S_WKV(float, 0, nseq, nullptr, nullptr, nullptr);
+    else K8S_WKV(bf16_t, 0, nseq, nullptr, nullptr, nullptr);
+    return (int)hipGetLastError();
   }
+  const int chunks = (T + Lc - 1) / Lc + nseq;
+  float* loc = ws;
+  float* start = ws + (size_t)chunks * H * D * D;
+  float* dec = start + (size_t)chunks * H * D * D;
+  if (f32) K8S_WKV(float, 1, chunks, loc, dec, nullptr);
+  else K8S_WKV(bf16_t, 1, chunks, loc, dec, nullptr);
+  wkv_prefix_kernel<<<dim3(nseq, H), 256, 0, s>>>(start, loc, dec, state, cu_q, seq_slots, positions, H, D, Lc);
+  if (f32) K8S_WKV(float, 2, chunks, nullptr, nullptr, start);
+  else K8S_WKV(bf16_t, 2, chunks, nullptr, nullptr, start);
 #undef K8S_WKV
   return (int)hipGetLastError();
 }

@@ -200,9 +200,15 @@ def wkv_max_dim() -> int:
     return 128
 
 
+# Batches of at least WKV_CHUNK_MIN tokens run the recurrence as three passes over chunks of WKV_CHUNK tokens (parallel
+# over chunks); shorter ones (decoding, short portions) as one workgroup per sequence.
+WKV_CHUNK = int(os.environ.get("K8S_WKV_CHUNK", "64"))
+WKV_CHUNK_MIN = int(os.environ.get("K8S_WKV_CHUNK_MIN", "256"))
+
+
 def wkv_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, z: torch.Tensor, w0: torch.Tensor,
              u: torch.Tensor, lnw: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor, seq_slots: torch.Tensor,
-             positions: torch.Tensor, H: int, D: int, eps: float) -> torch.Tensor:
+             positions: torch.Tensor, H: int, D: int, eps: float, chunk: Optional[int] = None) -> torch.Tensor:
     """The recurrence with its per-head unit norm, norm weight and silu gate; r, k, v, g [T, H D] (one row stride),
     z [T, H D] fp32 decay logits (w = exp(-exp(z + w0))), ``state`` [slots, H, D, D] fp32 updated in place."""
     T = r.shape[0]
@@ -217,10 +223,13 @@ def wkv_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor,
         if t.stride(0) != ld or t.stride(1) != 1 or t.dtype != r.dtype:
             raise ValueError("wkv_scan: r, k, v, g must share dtype and row stride")
     out = torch.empty(T, H * D, dtype=r.dtype, device=r.device)
+    nseq = cu_q.shape[0] - 1
+    Lc = (WKV_CHUNK if T >= WKV_CHUNK_MIN else 0) if chunk is None else int(chunk)
+    ws = torch.empty(_native().wkv_workspace(T, nseq, H, D, Lc), dtype=F32, device=r.device) if Lc > 0 else None
     _native().wkv_scan(out.data_ptr(), r.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), ld, _p(z),
                        _p(w0, r.dtype, "w0"), _p(u, r.dtype, "u"), _p(lnw, r.dtype, "lnw"), _p(state),
-                       _p(cu_q, I32), _p(seq_slots, I32), _p(positions, I32), cu_q.shape[0] - 1, H, D, float(eps),
-                       _f32(r.dtype), -1)
+                       _p(cu_q, I32), _p(seq_slots, I32), _p(positions, I32), nseq, H, D, float(eps),
+                       _f32(r.dtype), T, Lc, _p(ws), -1)
     return out
 
 

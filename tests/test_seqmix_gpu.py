@@ -107,6 +107,13 @@ def test_wkv_scan(dt, tol, H, D):
     close(og, oc, tol * 3)
     close(Sg, Sc, 1e-4)
     assert torch.equal(Sg[1].cpu(), S[1])        # the empty sequence's slot is untouched
+    for chunk in (4, 5, 16, 64):                  # the three-pass form over chunks: the same outputs and end states
+        Sk = S.to(DEV).clone()
+        ok = sm.wkv_scan(*(t.to(DEV) for t in (r, k, v, g, z, w0, u, lnw)), Sk, cu.to(DEV), slots.to(DEV), pos.to(DEV), H, D,
+                         1e-6, chunk=chunk)
+        close(ok, oc, tol * 3)
+        close(Sk, Sc, 1e-4)
+        assert torch.equal(Sk[1].cpu(), S[1])
 
 
 @pytest.mark.parametrize("dt,tol", DTYPES)
