@@ -136,7 +136,8 @@ int k8s_latent_attention(void* out, const void* q_abs, const void* q, const void
 int k8s_latent_mfma_ok(int C, int R, int Dn);
 int k8s_latent_attention_mfma(void* out, float* pacc, float* pml, const void* q_abs, const void* q, const void* cache,
                               const int* block_tables, int max_blocks, const int* tok_seq, const int* positions, int T,
-                              int C, int R, int H, int Dn, int window, float scale, int bs, int nsplit, hipStream_t s);
+                              int C, int R, int H, int Dn, int window, float scale, int bs, int nsplit, const int* cu_q,
+                              int nseq, int max_qlen, hipStream_t s);
 int k8s_moe_route(int* idx, float* w, const float* logits, int ld, int T, int E, int top, float scale, hipStream_t s);
 int k8s_moe_align(int* sorted_tok, int* pos_of_pair, int* seg, int* tiles, int ntiles, const int* topk_idx, int P,
                   int top, int E, int BM, hipStream_t s);
@@ -435,10 +436,10 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
   m.def("latent_attention_mfma", [](uintptr_t out, uintptr_t pacc, uintptr_t pml, uintptr_t q_abs, uintptr_t q,
                                     uintptr_t cache, uintptr_t bt, int max_blocks, uintptr_t tok_seq,
                                     uintptr_t positions, int T, int C, int R, int H, int Dn, int window, float scale,
-                                    int bs, int nsplit, int64_t s) {
+                                    int bs, int nsplit, uintptr_t cu_q, int nseq, int max_qlen, int64_t s) {
     check(k8s_latent_attention_mfma(P(out), P<float>(pacc), P<float>(pml), P(q_abs), P(q), P(cache), P<int>(bt),
                                     max_blocks, P<int>(tok_seq), P<int>(positions), T, C, R, H, Dn, window, scale, bs,
-                                    nsplit, S(s)), "latent_attention_mfma");
+                                    nsplit, P<int>(cu_q), nseq, max_qlen, S(s)), "latent_attention_mfma");
   });
   m.def("moe_route", [](uintptr_t idx, uintptr_t w, uintptr_t logits, int ld, int T, int E, int top, float scale,
                         int64_t s) {

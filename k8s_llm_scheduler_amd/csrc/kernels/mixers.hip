@@ -373,77 +373,104 @@ __global__ void latent_attention_kernel(TA* __restrict__ out, const TA* __restri
 // splits > 1 (few tokens: decoding) every split writes (max, sum, unnormalised O) and latent_merge_kernel joins them.
 typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
 
-template <int NDB>
-__global__ __launch_bounds__(64) void latent_attention_mfma_kernel(
+// NWV = 1: one wave per (token, head group, key split) -- decoding, where every token is another sequence.
+// NWV = 4: one workgroup per (4 consecutive tokens of a sequence, head group); the waves share every staged key step
+// (the union of their windows) and mask their own range, so a prompt reads each cached row once per 4 queries.
+// The queries stay in registers (NKK 32-wide pieces of [q_abs | q_rot] per lane).
+template <int NDB, int NKK, int NWV>
+__global__ __launch_bounds__(64 * NWV) void latent_attention_mfma_kernel(
     bf16_t* __restrict__ out, float* __restrict__ pacc, float* __restrict__ pml, const bf16_t* __restrict__ q_abs,
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache, const int* __restrict__ block_tables, int max_blocks,
-    const int* __restrict__ tok_seq, const int* __restrict__ positions, int C, int R, int H, int Dn, int window,
-    float scale, int bs, int nsplit) {
+    const int* __restrict__ tok_seq, const int* __restrict__ positions, const int* __restrict__ cu_q, int C, int R,
+    int H, int Dn, int window, float scale, int bs, int nsplit) {
   extern __shared__ __attribute__((aligned(16))) char smem_b[];
-  char* smem = smem_b;
-  const int t = blockIdx.x, hg = blockIdx.y, split = blockIdx.z;
-  const int lane = threadIdx.x, li = lane & 15, g = lane >> 4;
+  char* klds = smem_b;               // [32][L + 8] bf16
+  const int hg = blockIdx.y;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 15, g = lane >> 4;
   const int L = C + R, rowb = (L + 8) * 2, ndb = C / 16, HP = gridDim.y * 16;
-  const int p = positions[t];
-  if (p < 0) {
-    if (nsplit == 1)
+  int t, split, seq, p_first, p_last;
+  bool valid;
+  if (NWV == 1) {
+    t = blockIdx.x;
+    split = blockIdx.z;
+    seq = tok_seq[t];
+    p_first = p_last = positions[t];
+    valid = true;
+  } else {
+    seq = blockIdx.z;
+    split = 0;
+    const int tq0 = cu_q[seq] + blockIdx.x * NWV, tend = cu_q[seq + 1];
+    if (tq0 >= tend) return;
+    const int nval = min(NWV, tend - tq0);
+    t = tq0 + wave;
+    valid = wave < nval;
+    p_first = positions[tq0];
+    p_last = p_first + nval - 1;
+  }
+  const int p = valid ? p_first + (NWV == 1 ? 0 : wave) : -1;
+  if (p_first < 0) {                 // idle rows: defined output
+    if (nsplit == 1 && valid)
       for (int i = lane; i < 16 * C; i += 64) {
         const int hd = hg * 16 + i / C;
         if (hd < H) out[((size_t)t * H + hd) * C + i % C] = 0;
       }
     return;
   }
-  char* qlds = smem;                 // [16][L + 8] bf16
-  char* klds = smem + 16 * rowb;     // [32][L + 8] bf16
+  const int lo_min = window > 0 ? max(0, p_first - window + 1) : 0;
   const int lo = window > 0 ? max(0, p - window + 1) : 0;
-  const int ntiles = (p + 1 - lo + 31) / 32;
+  const int ntiles = (p_last + 1 - lo_min + 31) / 32;
   const int tps = (ntiles + nsplit - 1) / nsplit;
   const int t0 = split * tps, t1 = min(ntiles, t0 + tps);
-  const int* btr = block_tables + (size_t)tok_seq[t] * max_blocks;
+  const int* btr = block_tables + (size_t)seq * max_blocks;
   const int cpr = L / 8;             // 16-byte chunks per row
   const u32x4 zero = u32x4{0u, 0u, 0u, 0u};
-  for (int idx = lane; idx < 16 * cpr; idx += 64) {
-    const int r = idx / cpr, c = idx - r * cpr, hd = hg * 16 + r;
-    u32x4 v = zero;
-    if (hd < H)
-      v = 8 * c < C ? *reinterpret_cast<const u32x4*>(q_abs + ((size_t)t * H + hd) * C + 8 * c)
-                    : *reinterpret_cast<const u32x4*>(q + ((size_t)t * H + hd) * (Dn + R) + Dn + (8 * c - C));
-    *reinterpret_cast<u32x4*>(qlds + r * rowb + 16 * c) = v;
+  const int nkk = (L + 31) / 32;
+  // B operand of S^T = K Q^T: lane (li = head, g) holds q[head][32 kk + 8 g .. + 7]
+  bf16x8 qf[NKK];
+  {
+    const int hd = hg * 16 + li;
+    const bool qok = valid && hd < H;
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {
+      const int piece = 32 * kk + 8 * g;
+      u32x4 v = zero;
+      if (qok && piece < L)
+        v = piece < C ? *reinterpret_cast<const u32x4*>(q_abs + ((size_t)t * H + hd) * C + piece)
+                      : *reinterpret_cast<const u32x4*>(q + ((size_t)t * H + hd) * (Dn + R) + Dn + (piece - C));
+      qf[kk] = __builtin_bit_cast(bf16x8, v);
+    }
   }
   f32x4 o[NDB];
 #pragma unroll
   for (int n = 0; n < NDB; ++n) o[n] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;
-  const int nkk = (L + 31) / 32;
   const int qd = li >> 2, pd = li & 3;
   for (int tile = t0; tile < t1; ++tile) {
-    const int j0 = lo + tile * 32;
+    const int j0 = lo_min + tile * 32;
     __syncthreads();
-    for (int idx = lane; idx < 32 * cpr; idx += 64) {
+    for (int idx = tid; idx < 32 * cpr; idx += 64 * NWV) {
       const int r = idx / cpr, c = idx - r * cpr, key = j0 + r;
       u32x4 v = zero;
-      if (key <= p) {
+      if (key <= p_last) {
         const size_t slot = (size_t)btr[key / bs] * bs + (key % bs);
         v = *reinterpret_cast<const u32x4*>(cache + slot * L + 8 * c);
       }
       *reinterpret_cast<u32x4*>(klds + r * rowb + 16 * c) = v;
     }
     __syncthreads();
+    if (!valid || j0 > p || j0 + 31 < lo) continue;     // no key of this step is visible to this wave's token
     f32x4 sacc[2];
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
       f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-      for (int kk = 0; kk < nkk; ++kk) {
-        const int piece = 32 * kk + 8 * g;
-        bf16x8 ka, qb;
-        if (piece < L) {
-          ka = *reinterpret_cast<const bf16x8*>(klds + (16 * m + li) * rowb + 2 * piece);
-          qb = *reinterpret_cast<const bf16x8*>(qlds + li * rowb + 2 * piece);
-        } else {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) { ka[e] = (__bf16)0.f; qb[e] = (__bf16)0.f; }
+      for (int kk = 0; kk < NKK; ++kk) {
+        if (kk < nkk) {
+          const int piece = 32 * kk + 8 * g;
+          bf16x8 ka = __builtin_bit_cast(bf16x8, zero);
+          if (piece < L) ka = *reinterpret_cast<const bf16x8*>(klds + (16 * m + li) * rowb + 2 * piece);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[kk], acc, 0, 0, 0);
         }
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb, acc, 0, 0, 0);
       }
       sacc[m] = acc;   // S[key j0 + 16 m + 4 g + i][head li]
     }
@@ -453,13 +480,13 @@ __global__ __launch_bounds__(64) void latent_attention_mfma_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int key = j0 + 16 * m + 4 * g + i;
-        const float v = key <= p ? sacc[m][i] * scale : -INFINITY;
+        const float v = (key <= p && key >= lo) ? sacc[m][i] * scale : -INFINITY;
         sacc[m][i] = v;
         tmax = fmaxf(tmax, v);
       }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
-    const float m_new = fmaxf(m_run, tmax);       // finite: key j0 is always visible
+    const float m_new = fmaxf(m_run, tmax);       // finite: the step holds a visible key
     const float alpha = m_run == -INFINITY ? 0.f : expf(m_run - m_new);
     float rsum = 0.f;
 #pragma unroll
@@ -499,6 +526,7 @@ __global__ __launch_bounds__(64) void latent_attention_mfma_kernel(
       }
     }
   }
+  if (!valid) return;
   // o[n][i] = O[head 4 g + i][d 16 n + li]; the head's (max, sum) live in the lanes with li == head
   float l_i[4], m_i[4];
 #pragma unroll
@@ -672,22 +700,38 @@ extern "C" int k8s_latent_attention(void* out, const void* q_abs, const void* q,
 // Whether the MFMA kernel takes these sizes (else the caller uses k8s_latent_attention).
 extern "C" int k8s_latent_mfma_ok(int C, int R, int Dn) {
   const int L = C + R;
-  return C % 16 == 0 && R % 8 == 0 && Dn % 8 == 0 && C <= 512 && 48 * (L + 8) * 2 <= 64 * 1024;
+  return C % 16 == 0 && R % 8 == 0 && Dn % 8 == 0 && C <= 512 && L <= 640;
 }
 
+// nsplit == 1 and cu_q given (nseq sequences of at most max_qlen tokens): 4 consecutive tokens of a sequence per
+// workgroup; else one wave per (token, head group, key split).
 extern "C" int k8s_latent_attention_mfma(void* out, float* pacc, float* pml, const void* q_abs, const void* q,
                                          const void* cache, const int* block_tables, int max_blocks,
                                          const int* tok_seq, const int* positions, int T, int C, int R, int H, int Dn,
-                                         int window, float scale, int bs, int nsplit, hipStream_t s) {
+                                         int window, float scale, int bs, int nsplit, const int* cu_q, int nseq,
+                                         int max_qlen, hipStream_t s) {
   if (T <= 0) return 0;
   if (!k8s_latent_mfma_ok(C, R, Dn) || H <= 0 || bs <= 0 || nsplit < 1 || (nsplit > 1 && (!pacc || !pml))) return -1;
   const int L = C + R, HG = (H + 15) / 16;
-  const size_t lds = (size_t)48 * (L + 8) * 2;
-  const dim3 grid(T, HG, nsplit);
-#define K8S_LM(NDB)   latent_attention_mfma_kernel<NDB><<<grid, 64, lds, s>>>((bf16_t*)out, pacc, pml, (const bf16_t*)q_abs,                                                           (const bf16_t*)q, (const bf16_t*)cache, block_tables,                                                           max_blocks, tok_seq, positions, C, R, H, Dn, window, scale,                                                           bs, nsplit)
-  if (C <= 128) K8S_LM(8);
-  else if (C <= 256) K8S_LM(16);
-  else K8S_LM(32);
+  const size_t lds = (size_t)32 * (L + 8) * 2;
+  const bool tiles = nsplit == 1 && cu_q != nullptr && nseq > 0 && max_qlen > 1;
+  if (tiles && nseq > 65535) return -2;
+  const dim3 grid = tiles ? dim3((max_qlen + 3) / 4, HG, nseq) : dim3(T, HG, nsplit);
+#define K8S_LM(NDB, NKK)                                                                                              \
+  do {                                                                                                                \
+    if (tiles)                                                                                                        \
+      latent_attention_mfma_kernel<NDB, NKK, 4><<<grid, 256, lds, s>>>(                                               \
+          (bf16_t*)out, pacc, pml, (const bf16_t*)q_abs, (const bf16_t*)q, (const bf16_t*)cache, block_tables,        \
+          max_blocks, tok_seq, positions, cu_q, C, R, H, Dn, window, scale, bs, nsplit);                              \
+    else                                                                                                              \
+      latent_attention_mfma_kernel<NDB, NKK, 1><<<grid, 64, lds, s>>>(                                                \
+          (bf16_t*)out, pacc, pml, (const bf16_t*)q_abs, (const bf16_t*)q, (const bf16_t*)cache, block_tables,        \
+          max_blocks, tok_seq, positions, cu_q, C, R, H, Dn, window, scale, bs, nsplit);                              \
+  } while (0)
+  if (C <= 128 && L <= 256) K8S_LM(8, 8);
+  else if (C <= 256 && L <= 256) K8S_LM(16, 8);
+  else if (C <= 256) K8S_LM(16, 20);
+  else K8S_LM(32, 20);
 #undef K8S_LM
   if (nsplit > 1)
     latent_merge_kernel<<<dim3(T, H), 128, 0, s>>>((bf16_t*)out, pacc, pml, positions, C, H, HG * 16, nsplit);

@@ -519,7 +519,8 @@ class PutulornModel:
         q_abs = torch.empty(T, H, C, dtype=self.dtype, device=h.device)
         sm.gemm(q.view(T, H, Dn + R)[:, :, :Dn].permute(1, 0, 2), w.uk_t, out=q_abs.permute(1, 0, 2))
         lat = sm.latent_attention(q_abs, q, cache, b["block_tables"], b["tok_seq"], b["positions"], C, R, H, Dn,
-                                  m.window, m.scale, self.block_size, b.get("max_keys", 0))     # [T, H, C]
+                                  m.window, m.scale, self.block_size, b.get("max_keys", 0), b["cu_q"],
+                                  b.get("max_qlen", 0))                   # [T, H, C]
         a = torch.empty(T, H, V, dtype=self.dtype, device=h.device)
         sm.gemm(lat.permute(1, 0, 2), w.uv, out=a.permute(1, 0, 2))
         return sm.linear(a.view(T, H * V), w.o)
@@ -598,6 +599,7 @@ class PutulornModel:
         if seq_slots is None:
             raise ValueError("a stateful model needs the sequences' state slots")
         b = self.batch_meta(positions, slot_mapping, cu_q, block_tables, seq_slots)
+        b["max_qlen"] = int(max_qlen)
         return self._forward(ids, b, last_idx.long())
 
     def forward_decode(self, tokens, context_lens, block_tables, max_context, cascade=None) -> torch.Tensor:

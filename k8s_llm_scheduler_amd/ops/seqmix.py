@@ -261,9 +261,12 @@ def latent_splits(T: int, H: int, max_keys: int) -> int:
 
 def latent_attention(q_abs: torch.Tensor, q: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor,
                      tok_seq: torch.Tensor, positions: torch.Tensor, C: int, R: int, H: int, Dn: int, window: int,
-                     scale: float, block_size: int, max_keys: int = 0) -> torch.Tensor:
+                     scale: float, block_size: int, max_keys: int = 0, cu_q: Optional[torch.Tensor] = None,
+                     max_qlen: int = 0) -> torch.Tensor:
     """Sliding-window attention in the latent space over the paged cache; returns softmax-weighted latents [T, H, C].
     ``max_keys``: an upper bound of the keys any token sees (sizes the key splits; 0: the table's capacity).
+    ``cu_q`` / ``max_qlen`` (the sequences' query offsets and longest portion): portions of prompts run four
+    consecutive tokens per workgroup, sharing the staged cache rows.
     bf16 with 16-byte-aligned parts runs on the matrix cores; fp32 and other sizes on the plain-FMA kernel."""
     if not _gpu(q_abs, q, cache):
         return ref.latent_attention(q_abs, q, cache, block_tables, tok_seq, positions, C, R, H, Dn, window, scale,
@@ -284,7 +287,9 @@ def latent_attention(q_abs: torch.Tensor, q: torch.Tensor, cache: torch.Tensor, 
             HP = (H + 15) // 16 * 16
             pacc = torch.empty(T * HP * ns * C, dtype=F32, device=q.device)
             pml = torch.empty(T * HP * ns * 2, dtype=F32, device=q.device)
-        nat.latent_attention_mfma(out.data_ptr(), _p(pacc), _p(pml), *args, ns, -1)
+        nseq = cu_q.shape[0] - 1 if cu_q is not None else 0
+        nat.latent_attention_mfma(out.data_ptr(), _p(pacc), _p(pml), *args, ns, _p(cu_q, I32, "cu_q"), nseq,
+                                  int(max_qlen), -1)
     else:
         nat.latent_attention(out.data_ptr(), *args, _f32(dt), -1)
     return out

@@ -139,10 +139,11 @@ def test_latent_attention(dt, tol, H, Dn, R, C, dims, win):
     close(cg, cc, tol)
     close(qg, qc, tol)
     qabs = torch.randn(T, H, C).to(dt) * 0.3
-    og = sm.latent_attention(qabs.to(DEV), qc.to(DEV), cc.to(DEV), bt.to(DEV), tok_seq.to(DEV), pos.to(DEV), C, R, H, Dn,
-                             win, 0.2, bs)
     oc = sm.latent_attention(qabs, qc, cc, bt, tok_seq, pos, C, R, H, Dn, win, 0.2, bs)
-    close(og, oc, tol)
+    for kw in ({}, {"cu_q": cu.to(DEV), "max_qlen": 27}):      # per token, and four tokens of a sequence per workgroup
+        og = sm.latent_attention(qabs.to(DEV), qc.to(DEV), cc.to(DEV), bt.to(DEV), tok_seq.to(DEV), pos.to(DEV), C, R, H,
+                                 Dn, win, 0.2, bs, **kw)
+        close(og, oc, tol)
 
 
 @pytest.mark.parametrize("dt,tol", DTYPES)
