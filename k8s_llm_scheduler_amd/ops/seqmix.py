@@ -95,7 +95,9 @@ def act(x: torch.Tensor, kind: int, limit: float = 0.0, alpha: float = 1.0) -> t
 
 
 def _route_fast(a: torch.Tensor, w: torch.Tensor, out_dtype) -> bool:
-    """bf16 products whose shape the framework's tuned GEMV / MFMA GEMM kernels take (128-byte k steps, N % 4 == 0)."""
+    """bf16 products of production size whose shape the framework's tuned GEMV / MFMA GEMM kernels take (128-byte
+    k steps, N % 16 == 0, at least 1024 x 512 weights: the sizes their plan tables and heuristics were tuned and
+    tested on).  Smaller products are launch-bound and stay on the any-shape kernel."""
     from . import GEMM_BACKEND
 
     if a.dtype != BF16 or w.dtype != BF16 or out_dtype not in (BF16, F32) or a.dim() != 2 or w.dim() != 2:
@@ -103,7 +105,7 @@ def _route_fast(a: torch.Tensor, w: torch.Tensor, out_dtype) -> bool:
     if GEMM_BACKEND == "library" or not a.is_contiguous() or not w.is_contiguous():
         return False
     N, K = w.shape
-    return K % 64 == 0 and N % 16 == 0 and K >= 128 and N >= 64
+    return K % 64 == 0 and N % 16 == 0 and K * N >= 512 * 1024 and K >= 128 and N >= 128
 
 
 # route fitting bf16 shapes to ops.linear (K8S_SEQMIX_FAST_GEMM=0: every product on the any-shape kernel)
@@ -117,9 +119,12 @@ def linear(a: torch.Tensor, w: torch.Tensor, out_dtype=None) -> torch.Tensor:
     if not _gpu(a, w):
         return ref.gemm_any(a, w, out_dtype)
     if FAST_GEMM and _route_fast(a, w, out_dtype):
-        from . import linear as tuned
+        from . import NoKernelForShape, linear as tuned
 
-        return tuned(a, w, out_dtype=F32 if out_dtype == F32 else None)
+        try:
+            return tuned(a, w, out_dtype=F32 if out_dtype == F32 else None)
+        except NoKernelForShape:
+            pass
     return gemm(a, w, out_dtype)
 
 
