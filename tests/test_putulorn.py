@@ -359,3 +359,45 @@ def test_greedy_generation_through_the_scheduler(tmp_path, device):
     if device == "cuda":
         assert eng.stats["graph_replays"] > 0
     assert len(eng.free_slots) == 2 and eng.allocator.num_free == eng.num_blocks
+
+
+# ----------------------------------------------------------------------------- command line
+def test_replay_and_generate_command_line(tmp_path):
+    """The replay runner as a user starts it: steps on standard input, one logits file per step that wants rows,
+    `done <step>` after every step; and `generate` on token ids."""
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    import numpy as np
+
+    root = Path(__file__).resolve().parent.parent
+    cfg = config([with_mlp(latent(), dense()), with_mlp(wkv(), moe())], loop=(0, 2, 2))
+    pc = config_from_json(cfg, "cli")
+    tensors = random_tensors(pc, 5)
+    save_checkpoint(pc, tensors, tmp_path / "ckpt")
+    a, b = tokens(21, cfg["vocab"], 70), tokens(9, cfg["vocab"], 71)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:17], "want": [0, 16]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[17:18], "want": []}, {"id": "b", "tokens": b, "want": [8]}],
+              "end": ["b"]},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[18:], "want": [2]}], "end": ["a"]}]
+    out = tmp_path / "out"
+    r = subprocess.run([str(root / "bin" / "trace_run"), "--model", str(tmp_path / "ckpt"), "--dtype", "float32", "--out",
+                        str(out), "--max-tokens", "64", "--device", "cpu"], input="\n".join(map(json.dumps, steps)) + "\n",
+                       capture_output=True, text=True, timeout=300, cwd=str(root))
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    assert sorted(p.name for p in out.iterdir()) == ["0.f32", "1.f32", "2.f32"]
+    wa, wb = oracle.forward(cfg, tensors, a), oracle.forward(cfg, tensors, b)
+    V = cfg["vocab"]
+    got = {i: torch.from_numpy(np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, V)) for i in range(3)}
+    assert rel_err(got[0], wa[[0, 16]]) < TOL["float32"]
+    assert rel_err(got[1], wb[[8]]) < TOL["float32"]
+    assert rel_err(got[2], wa[[20]]) < TOL["float32"]
+    g = subprocess.run([sys.executable, "-m", "k8s_llm_scheduler_amd", "generate", "--model", str(tmp_path / "ckpt"),
+                        "--dtype", "float32", "--prompt", " ".join(map(str, b)), "--max-new", "5", "--device", "cpu",
+                        "--no-graphs"], capture_output=True, text=True, timeout=300, cwd=str(root))
+    assert g.returncode == 0, g.stderr[-2000:]
+    line = json.loads([l for l in g.stdout.splitlines() if l.startswith("{")][-1])
+    assert line["token_ids"] == oracle.greedy(cfg, tensors, b, 5)
