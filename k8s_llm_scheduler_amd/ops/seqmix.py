@@ -131,9 +131,11 @@ def linear(a: torch.Tensor, w: torch.Tensor, out_dtype=None) -> torch.Tensor:
 def gemm(a: torch.Tensor, w: torch.Tensor, out_dtype=None, *, a_rows: Optional[torch.Tensor] = None,
          tiles: Optional[torch.Tensor] = None, rows: Optional[int] = None,
          seg: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """The any-shape GEMM.  2-D: a [M, K] (row stride free) @ w [N, K]^T.  3-D: batched over dim 0 (a [G, M, K] with any
-    strides whose last is 1, w [G, N, K]) -> [G, M, N] (``out``: a [G, M, N] view with any batch / row strides).  Grouped (``tiles`` [n, 3] from :func:`moe_align`, w [G, N, K]):
-    ``rows`` compact rows, row r = a[a_rows[r]] (or a[r]), the rows of tile (g, r0, n) use w[g] -> [rows, N]."""
+    """The any-shape GEMM.  2-D: a [M, K] (row stride free) @ w [N, K]^T.  3-D: batched over dim 0 (a [G, M, K] with
+    any strides whose last is 1, w [G, N, K]) -> [G, M, N]; ``out``: a [G, M, N] view with any batch / row strides.
+    Grouped (``tiles`` [n, 3] from :func:`moe_align`, w [G, N, K]): ``rows`` compact rows, row r = a[a_rows[r]] (or
+    a[r]), the rows of tile (g, r0, n) use w[g] -> [rows, N] (``seg``: the groups' row offsets, read by the CPU
+    reference only)."""
     out_dtype = out_dtype or a.dtype
     if a.dtype != w.dtype:
         raise TypeError(f"gemm operands differ in dtype: {a.dtype} and {w.dtype}")
