@@ -401,3 +401,67 @@ def test_replay_and_generate_command_line(tmp_path):
     assert g.returncode == 0, g.stderr[-2000:]
     line = json.loads([l for l in g.stdout.splitlines() if l.startswith("{")][-1])
     assert line["token_ids"] == oracle.greedy(cfg, tensors, b, 5)
+
+
+# ----------------------------------------------------------------------------- random configurations
+def random_config(seed):
+    """A random small model: 2-5 layers of either mixer in any order, any feed-forward (or none), sizes that are and
+    are not multiples of 8 / 16, windows from 1 to beyond the sequence, an optional loop over any span."""
+    import random
+
+    rng = random.Random(seed)
+    aligned = rng.random() < 0.5
+    pick = lambda xs: rng.choice(xs)
+    width = pick([32, 64, 96]) if aligned else pick([24, 37, 50, 72])
+    layers = []
+    for _ in range(rng.randint(2, 5)):
+        if rng.random() < 0.5:
+            heads = pick([1, 2, 3, 4])
+            layer = wkv(heads=heads, dim=pick([8, 16, 32]) if aligned else pick([5, 12, 20, 33]))
+        else:
+            rd = pick([0, 8, 16]) if aligned else pick([0, 2, 6, 10])
+            layer = latent(heads=pick([1, 2, 5, 17]), dim=pick([8, 16, 24]) if aligned else pick([3, 10, 12]),
+                           rot_dim=rd, vdim=pick([8, 16]) if aligned else pick([5, 9]),
+                           kv_rank=pick([16, 32, 48]) if aligned else pick([7, 20, 36]),
+                           window=pick([0, 1, 2, 7, 31, 32, 33, 50, 500]), dims=pick([rd, rd // 2 * 2 // 2 * 2, rd]),
+                           base=pick([100.0, 10000.0, 1e6]), scale=pick([0.1, 0.25, 0.5]))
+        r = rng.random()
+        if r < 0.35:
+            layer = with_mlp(layer, dense(pick([16, 40, 64]) if aligned else pick([10, 27])))
+        elif r < 0.8:
+            e = pick([2, 3, 8, 20])
+            layer = with_mlp(layer, moe(experts=e, top=rng.randint(1, min(e, 4)), ff=pick([8, 16]) if aligned else pick([5, 12]),
+                                        scale=pick([0.5, 1.0, 2.5]), limit=pick([0, 0.7, 3.0]), shared=rng.random() < 0.6,
+                                        shared_limit=pick([0, 1.5])))
+        layers.append(layer)
+    loop = None
+    if rng.random() < 0.6:
+        a = rng.randrange(len(layers))
+        loop = (a, rng.randint(a + 1, len(layers)), rng.randint(1, 3))
+    return config(layers, width=width, vocab=pick([40, 64, 101]), loop=loop, mult=pick([0.3, 0.7, 1.0]),
+                  eps=pick([1e-6, 1e-5]))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("seed", range(8))
+def test_random_configurations(tmp_path, device, seed):
+    """A prompt in two portions, a second request beside its decoded tokens, then tokens one by one."""
+    cfg = random_config(seed)
+    eng, tensors = make(tmp_path, cfg, device, "float32", seed=seed, max_tokens=160, slots=2)
+    V = cfg["vocab"]
+    a, b = tokens(75, V, 100 + seed), tokens(28, V, 200 + seed)
+    wa, wb = oracle.forward(cfg, tensors, a), oracle.forward(cfg, tensors, b)
+    ga = [eng.replay_step([("a", a[:40], list(range(40)))]), eng.replay_step([("a", a[40:43], [0, 1, 2])])]
+    gb = []
+    for i in range(43, 75):
+        if i == 50:
+            rows = eng.replay_step([("a", [a[i]], [0]), ("b", b[:20], list(range(20)))])
+            gb.append(rows[1:])
+        elif 50 < i <= 58:
+            rows = eng.replay_step([("a", [a[i]], [0]), ("b", [b[20 + i - 51]], [0])], ["b"] if i == 58 else [])
+            gb.append(rows[1:])
+        else:
+            rows = eng.replay_step([("a", [a[i]], [0])])
+        ga.append(rows[:1])
+    assert rel_err(torch.cat(ga), wa) < TOL["float32"], cfg
+    assert rel_err(torch.cat(gb), wb) < TOL["float32"], cfg
