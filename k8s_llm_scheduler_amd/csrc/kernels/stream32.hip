@@ -150,16 +150,18 @@ __global__ __launch_bounds__(256) void gemm_any_kernel(TO* __restrict__ C, const
 }
 
 // The same product for bf16 operands whose rows are 16-byte aligned (k and every stride a multiple of 8 elements) on
-// the matrix cores: 64 x 64 output tile, 32-deep k steps, 4 waves of 32 x 32 (2 x 2 v_mfma_f32_16x16x32_bf16) in the
-// swapped orientation C^T = W A^T, so a lane ends with 4 consecutive columns of one row.  The next k step's global
+// the matrix cores: 64 x 64 or (many rows and columns) 64 x 128 output tile, 32-deep k steps, 4 waves of 32 x 32 or
+// 32 x 64 (2 x NF v_mfma_f32_16x16x32_bf16) in the swapped orientation C^T = W A^T, so a lane ends with 4 consecutive
+// columns of one row; an output's accumulation is the same in both tile shapes.  The next k step's global
 // loads are in flight during the current step's MFMAs.  Same three forms (batched, row gather, grouped tiles); the
 // accumulation order of an output does not depend on M or on the rows that share its tile.
-template <typename TO>
+template <typename TO, int NF>   // NF 16-column fragments per wave: output tile 64 x (32 NF)
 __global__ __launch_bounds__(256) void gemm_mfma_kernel(TO* __restrict__ C, const bf16_t* __restrict__ A,
                                                         const bf16_t* __restrict__ Wt, int M, int N, int K, long lda,
                                                         long ldw, long ldc, long sA, long sW, long sC,
                                                         const int* __restrict__ a_rows, const int* __restrict__ tiles) {
-  constexpr int BM = 64, BN = 64, BK = 32, LDK = BK + 8;   // rows of 80 bytes: 16-byte aligned fragments
+  constexpr int BM = 64, BN = 32 * NF, BK = 32, LDK = BK + 8;   // rows of 80 bytes: 16-byte aligned fragments
+  constexpr int WL = BN / 64;                                    // W rows per loader thread
   __shared__ __attribute__((aligned(16))) bf16_t As[BM][LDK];
   __shared__ __attribute__((aligned(16))) bf16_t Ws[BN][LDK];
   int row0, rows;
@@ -178,40 +180,48 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(TO* __restrict__ C, cons
   }
   const int col0 = blockIdx.x * BN;
   const int tid = threadIdx.x;
-  // loader: thread -> (row tid / 4, 8-element chunk tid % 4) of both tiles
+  // loader: thread -> (row tid / 4 (+ 64 c for W), 8-element chunk tid % 4)
   const int lr = tid >> 2, lc = tid & 3;
-  const bool a_ok = lr < rows, w_ok = col0 + lr < N;
+  const bool a_ok = lr < rows;
   const int gr = a_ok ? (a_rows != nullptr ? a_rows[row0 + lr] : row0 + lr) : 0;
   const bf16_t* ap = A + (size_t)gr * lda + lc * 8;
-  const bf16_t* wp = Wt + (size_t)(w_ok ? col0 + lr : 0) * ldw + lc * 8;
+  const bf16_t* wp[WL];
+  bool w_ok[WL];
+#pragma unroll
+  for (int c = 0; c < WL; ++c) {
+    w_ok[c] = col0 + lr + 64 * c < N;
+    wp[c] = Wt + (size_t)(w_ok[c] ? col0 + lr + 64 * c : 0) * ldw + lc * 8;
+  }
   const u32x4 zero = u32x4{0u, 0u, 0u, 0u};
-  u32x4 ra, rw;
+  u32x4 ra, rw[WL];
   auto fetch = [&](int k0) {
     const bool kin = k0 + lc * 8 < K;
     ra = (kin && a_ok) ? *reinterpret_cast<const u32x4*>(ap + k0) : zero;
-    rw = (kin && w_ok) ? *reinterpret_cast<const u32x4*>(wp + k0) : zero;
+#pragma unroll
+    for (int c = 0; c < WL; ++c) rw[c] = (kin && w_ok[c]) ? *reinterpret_cast<const u32x4*>(wp[c] + k0) : zero;
   };
   const int lane = tid & 63, wave = tid >> 6, li = lane & 15, g = lane >> 4;
-  const int m0 = (wave & 1) * 32, n0 = (wave >> 1) * 32;
-  f32x4 acc[2][2];
+  const int m0 = (wave & 1) * 32, n0 = (wave >> 1) * (16 * NF);
+  f32x4 acc[NF][2];
 #pragma unroll
-  for (int f = 0; f < 2; ++f)
+  for (int f = 0; f < NF; ++f)
 #pragma unroll
     for (int j = 0; j < 2; ++j) acc[f][j] = f32x4{0.f, 0.f, 0.f, 0.f};
   fetch(0);
   for (int k0 = 0; k0 < K; k0 += BK) {
     __syncthreads();
     *reinterpret_cast<u32x4*>(&As[lr][lc * 8]) = ra;
-    *reinterpret_cast<u32x4*>(&Ws[lr][lc * 8]) = rw;
+#pragma unroll
+    for (int c = 0; c < WL; ++c) *reinterpret_cast<u32x4*>(&Ws[lr + 64 * c][lc * 8]) = rw[c];
     __syncthreads();
     if (k0 + BK < K) fetch(k0 + BK);
-    bf16x8 wf[2], af[2];
+    bf16x8 wf[NF], af[2];
 #pragma unroll
-    for (int f = 0; f < 2; ++f) wf[f] = *reinterpret_cast<const bf16x8*>(&Ws[n0 + 16 * f + li][8 * g]);
+    for (int f = 0; f < NF; ++f) wf[f] = *reinterpret_cast<const bf16x8*>(&Ws[n0 + 16 * f + li][8 * g]);
 #pragma unroll
     for (int j = 0; j < 2; ++j) af[j] = *reinterpret_cast<const bf16x8*>(&As[m0 + 16 * j + li][8 * g]);
 #pragma unroll
-    for (int f = 0; f < 2; ++f)
+    for (int f = 0; f < NF; ++f)
 #pragma unroll
       for (int j = 0; j < 2; ++j) acc[f][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[f], af[j], acc[f][j], 0, 0, 0);
   }
@@ -221,7 +231,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(TO* __restrict__ C, cons
     const int r = m0 + 16 * j + li;
     if (r >= rows) continue;
 #pragma unroll
-    for (int f = 0; f < 2; ++f)
+    for (int f = 0; f < NF; ++f)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int c = col0 + n0 + 16 * f + 4 * g + i;
@@ -281,19 +291,21 @@ extern "C" int k8s_gemm_any(void* C, const void* A, const void* W, int M, int N,
     gy = (M + 63) / 64;
   }
   if (gy > 65535 || batch > 65535) return -2;
-  const dim3 grid((N + 63) / 64, gy, batch);
   // bf16 rows that can be moved as 16-byte vectors: the MFMA kernel; anything else (fp32, odd strides): plain FMAs
   const bool vec = !in_f32 && K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && sA % 8 == 0 && sW % 8 == 0 &&
                    ((uintptr_t)A & 15) == 0 && ((uintptr_t)W & 15) == 0;
   if (vec) {
-    if (out_f32)
-      gemm_mfma_kernel<float><<<grid, 256, 0, s>>>((float*)C, (const bf16_t*)A, (const bf16_t*)W, M, N, K, lda, ldw,
-                                                   ldc, sA, sW, sC, a_rows, tiles);
-    else
-      gemm_mfma_kernel<bf16_t><<<grid, 256, 0, s>>>((bf16_t*)C, (const bf16_t*)A, (const bf16_t*)W, M, N, K, lda, ldw,
-                                                    ldc, sA, sW, sC, a_rows, tiles);
+    const bool wide = N >= 512 && (long)gy * ((N + 127) / 128) * batch >= 256;   // enough 64 x 128 tiles for the chip
+    const dim3 g2((N + (wide ? 127 : 63)) / (wide ? 128 : 64), gy, batch);
+#define K8S_GM(TO, NF) \
+  gemm_mfma_kernel<TO, NF><<<g2, 256, 0, s>>>((TO*)C, (const bf16_t*)A, (const bf16_t*)W, M, N, K, lda, ldw, ldc, sA, \
+                                              sW, sC, a_rows, tiles)
+    if (out_f32) { if (wide) K8S_GM(float, 4); else K8S_GM(float, 2); }
+    else { if (wide) K8S_GM(bf16_t, 4); else K8S_GM(bf16_t, 2); }
+#undef K8S_GM
     return (int)hipGetLastError();
   }
+  const dim3 grid((N + 63) / 64, gy, batch);
 #define K8S_GA(TI, TO) \
   gemm_any_kernel<TI, TO><<<grid, 256, 0, s>>>((TO*)C, (const TI*)A, (const TI*)W, M, N, K, lda, ldw, ldc, sA, sW, sC, \
                                                a_rows, tiles)

@@ -52,7 +52,7 @@ def test_stream_ops(dt, tol):
 
 @pytest.mark.parametrize("dt,tol", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(37, 200, 96), (1, 16, 256), (130, 70, 16), (64, 64, 64), (5, 640, 255), (3, 7, 5),
-                                   (200, 136, 72), (65, 129, 1032)])
+                                   (200, 136, 72), (65, 129, 1032), (1100, 2056, 40), (2048, 1024, 64)])
 def test_gemm_shapes(dt, tol, M, N, K):
     torch.manual_seed(1)
     a, w = torch.randn(M, K).to(dt), (torch.randn(N, K) / K ** 0.5).to(dt)
@@ -199,3 +199,17 @@ def test_latent_attention_long_contexts(dt, tol, H, win):
         close(og.cpu()[live], oc[live], tol)
         assert torch.equal(og.cpu()[~live].float(), torch.zeros(1, H, C))
     assert sm.latent_splits(Tn, H, 512) > 1 and sm.latent_splits(4096, H, 512) == 1
+
+
+def test_grouped_gemm_many_rows():
+    """Enough row tiles for the wide (64 x 128) form of the MFMA GEMM, grouped by expert with gathered rows."""
+    torch.manual_seed(8)
+    Tn, top, E, N, K = 1500, 2, 4, 1032, 64
+    idx = torch.randint(0, E, (Tn, top), dtype=torch.int32)
+    st, pos, seg, tiles = sm.moe_align(idx.to(DEV), E)
+    stc, posc, segc, tilesc = sm.moe_align(idx, E)
+    h, w = torch.randn(Tn, K).to(torch.bfloat16), (torch.randn(E, N, K) / K ** 0.5).to(torch.bfloat16)
+    got = sm.gemm(h.to(DEV), w.to(DEV), a_rows=st, tiles=tiles, rows=Tn * top).cpu().float()
+    want = sm.gemm(h, w, a_rows=stc, tiles=tilesc, rows=Tn * top, seg=segc).float()
+    # rows of an expert may come in another order: compare per (token, choice) pair
+    close(got[pos.cpu().long()], want[posc.long()], 2e-2)
