@@ -493,7 +493,6 @@ class PutulornModel:
     # ------------------------------------------------------------------ layers
     def _wkv(self, w: _Wkv, run: _Run, h, b) -> torch.Tensor:
         m = w.cfg
-        T = h.shape[0]
         S, shift = self.states[run.cache]
         mix = sm.token_shift(h, w.mu, shift, b["cu_q"], b["tok_seq"], b["seq_slots"], b["positions"])   # [5, T, W]
         sm.shift_save(shift, h, b["cu_q"], b["seq_slots"], b["positions"])

@@ -3,7 +3,6 @@ against the plain float64 oracle in putulorn_oracle.py.  Every test runs on the 
 state and scheduler logic) and, marked gpu, on the HIP kernels.  Small own configurations, random weights."""
 
 import copy
-import math
 
 import pytest
 import torch
