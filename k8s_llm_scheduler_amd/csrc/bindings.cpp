@@ -110,10 +110,12 @@ int k8s_pgemm4_config(int cfg, int* bp, int* bq, int* lds_bytes);
 int k8s_pgemm4_plan(int M, int N_out, int K, int epi, int cfg, int splits, int* nwg, long long* slab_elems);
 int k8s_pgemm4(void* out, float* slab, const void* x, const void* W, int M, int N_out, int K, int epi, int cfg,
                int splits, int group_m, const void* res, int rms, float eps, hipStream_t s);
-int k8s_embed_rows(float* out, const int* ids, const void* table, int T, int W, int vocab, int f32, hipStream_t s);
+int k8s_embed_rows(float* out, const int* ids, const void* table, int T, int W, int vocab, float scale, int f32,
+                   hipStream_t s);
 int k8s_resnorm(float* x, const void* branch, float mult, const void* rowvec, const void* w, float offset, float eps,
-                void* out, int T, int W, int f32, hipStream_t s);
-int k8s_act(void* out, const void* x, int T, int F, int kind, float limit, float alpha, int f32, hipStream_t s);
+                void* out, int T, int W, int groups, int f32, hipStream_t s);
+int k8s_act(void* out, const void* x, int T, int F, int kind, float limit, float alpha, const float* row_scale,
+            const int* row_map, int f32, hipStream_t s);
 int k8s_gemm_any(void* C, const void* A, const void* W, int M, int N, int K, long lda, long ldw, long ldc, int batch,
                  long sA, long sW, long sC, const int* a_rows, const int* tiles, int ntiles, int in_f32, int out_f32,
                  hipStream_t s);
@@ -138,7 +140,25 @@ int k8s_latent_attention_mfma(void* out, float* pacc, float* pml, const void* q_
                               const int* block_tables, int max_blocks, const int* tok_seq, const int* positions, int T,
                               int C, int R, int H, int Dn, int window, float scale, int bs, int nsplit, const int* cu_q,
                               int nseq, int max_qlen, hipStream_t s);
-int k8s_moe_route(int* idx, float* w, const float* logits, int ld, int T, int E, int top, float scale, hipStream_t s);
+int k8s_moe_route(int* idx, float* w, const float* logits, int ld, int T, int E, int top, float scale, int mode,
+                  hipStream_t s);
+int k8s_window_kv_write(void* kcache, void* vcache, void* qkv, long ld, int koff, int voff, const void* qb,
+                        const void* kb, const void* vb, const float* cos_sin, const int* positions,
+                        const int* slot_mapping, const float* vfirst_in, float* vfirst_out, float lam, int T, int H, int G,
+                        int D, int V, int dims, float eps, int unit, int f32, hipStream_t s);
+int k8s_window_pool(float* kpool, float* vpool, const void* kcache, const void* vcache, const int* block_tables,
+                    int max_blocks, const int* tok_seq, const int* positions, int T, int G, int D, int V, int P, int bs,
+                    int f32, hipStream_t s);
+int k8s_window_attention(void* out, const void* q, long ldq, const void* gate, long ldg, const void* kcache,
+                         const void* vcache, const float* kpool, const float* vpool, const int* block_tables,
+                         int max_blocks, const int* tok_seq, const int* positions, int T, int H, int G, int D, int V,
+                         int window, int P, float scale, int sink, int bs, int f32, hipStream_t s);
+int k8s_gated_scan_max_dim();
+long long k8s_gated_scan_record(int kind, int D, int V);
+int k8s_gated_scan(void* out, const float* proj, long ld, int kind, int cq, int ck, int cv, int ci, int cf, int cg,
+                   const void* fbias, const void* ibias, const void* lower, const void* normw, float* state,
+                   const int* cu_q, const int* seq_slots, const int* positions, int nseq, int H, int D, int V, float eps,
+                   float cap, int f32, hipStream_t s);
 int k8s_moe_align(int* sorted_tok, int* pos_of_pair, int* seg, int* tiles, int ntiles, const int* topk_idx, int P,
                   int top, int E, int BM, hipStream_t s);
 int k8s_moe_combine(void* z, const void* D, const int* pos, const float* w, const void* shared, const float* logits,
@@ -384,15 +404,18 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
   });
 
   // fp32 residual stream, recurrent / latent mixers, mixture of experts (stream32.hip, mixers.hip, moe.hip)
-  m.def("embed_rows", [](uintptr_t out, uintptr_t ids, uintptr_t table, int T, int W, int vocab, int f32, int64_t s) {
-    check(k8s_embed_rows(P<float>(out), P<int>(ids), P(table), T, W, vocab, f32, S(s)), "embed_rows");
+  m.def("embed_rows", [](uintptr_t out, uintptr_t ids, uintptr_t table, int T, int W, int vocab, float scale, int f32,
+                         int64_t s) {
+    check(k8s_embed_rows(P<float>(out), P<int>(ids), P(table), T, W, vocab, scale, f32, S(s)), "embed_rows");
   });
   m.def("resnorm", [](uintptr_t x, uintptr_t branch, float mult, uintptr_t rowvec, uintptr_t w, float offset, float eps,
-                      uintptr_t out, int T, int W, int f32, int64_t s) {
-    check(k8s_resnorm(P<float>(x), P(branch), mult, P(rowvec), P(w), offset, eps, P(out), T, W, f32, S(s)), "resnorm");
+                      uintptr_t out, int T, int W, int groups, int f32, int64_t s) {
+    check(k8s_resnorm(P<float>(x), P(branch), mult, P(rowvec), P(w), offset, eps, P(out), T, W, groups, f32, S(s)),
+          "resnorm");
   });
-  m.def("act", [](uintptr_t out, uintptr_t x, int T, int F, int kind, float limit, float alpha, int f32, int64_t s) {
-    check(k8s_act(P(out), P(x), T, F, kind, limit, alpha, f32, S(s)), "act");
+  m.def("act", [](uintptr_t out, uintptr_t x, int T, int F, int kind, float limit, float alpha, uintptr_t row_scale,
+                  uintptr_t row_map, int f32, int64_t s) {
+    check(k8s_act(P(out), P(x), T, F, kind, limit, alpha, P<float>(row_scale), P<int>(row_map), f32, S(s)), "act");
   });
   m.def("gemm_any", [](uintptr_t C, uintptr_t A, uintptr_t W, int M, int N, int K, long lda, long ldw, long ldc,
                        int batch, long sA, long sW, long sC, uintptr_t a_rows, uintptr_t tiles, int ntiles, int in_f32,
@@ -442,8 +465,42 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
                                     nsplit, P<int>(cu_q), nseq, max_qlen, S(s)), "latent_attention_mfma");
   });
   m.def("moe_route", [](uintptr_t idx, uintptr_t w, uintptr_t logits, int ld, int T, int E, int top, float scale,
-                        int64_t s) {
-    check(k8s_moe_route(P<int>(idx), P<float>(w), P<float>(logits), ld, T, E, top, scale, S(s)), "moe_route");
+                        int mode, int64_t s) {
+    check(k8s_moe_route(P<int>(idx), P<float>(w), P<float>(logits), ld, T, E, top, scale, mode, S(s)), "moe_route");
+  });
+  // windowed grouped-query attention with pooled far blocks, gated matrix-state recurrences (window_attn.hip,
+  // gated_scan.hip)
+  m.def("window_kv_write", [](uintptr_t kcache, uintptr_t vcache, uintptr_t qkv, long ld, int koff, int voff,
+                              uintptr_t qb, uintptr_t kb, uintptr_t vb, uintptr_t cos_sin, uintptr_t positions,
+                              uintptr_t slots, uintptr_t vfirst_in, uintptr_t vfirst_out, float lam, int T, int H, int G,
+                              int D, int V, int dims, float eps, int unit, int f32, int64_t s) {
+    check(k8s_window_kv_write(P(kcache), P(vcache), P(qkv), ld, koff, voff, P(qb), P(kb), P(vb), P<float>(cos_sin),
+                              P<int>(positions), P<int>(slots), P<float>(vfirst_in), P<float>(vfirst_out), lam, T, H, G,
+                              D, V, dims, eps, unit, f32, S(s)), "window_kv_write");
+  });
+  m.def("window_pool", [](uintptr_t kpool, uintptr_t vpool, uintptr_t kcache, uintptr_t vcache, uintptr_t bt,
+                          int max_blocks, uintptr_t tok_seq, uintptr_t positions, int T, int G, int D, int V, int P_,
+                          int bs, int f32, int64_t s) {
+    check(k8s_window_pool(P<float>(kpool), P<float>(vpool), P(kcache), P(vcache), P<int>(bt), max_blocks,
+                          P<int>(tok_seq), P<int>(positions), T, G, D, V, P_, bs, f32, S(s)), "window_pool");
+  });
+  m.def("window_attention", [](uintptr_t out, uintptr_t q, long ldq, uintptr_t gate, long ldg, uintptr_t kcache,
+                               uintptr_t vcache, uintptr_t kpool, uintptr_t vpool, uintptr_t bt, int max_blocks,
+                               uintptr_t tok_seq, uintptr_t positions, int T, int H, int G, int D, int V, int window,
+                               int P_, float scale, int sink, int bs, int f32, int64_t s) {
+    check(k8s_window_attention(P(out), P(q), ldq, P(gate), ldg, P(kcache), P(vcache), P<float>(kpool), P<float>(vpool),
+                               P<int>(bt), max_blocks, P<int>(tok_seq), P<int>(positions), T, H, G, D, V, window, P_,
+                               scale, sink, bs, f32, S(s)), "window_attention");
+  });
+  m.def("gated_scan_max_dim", []() { return k8s_gated_scan_max_dim(); });
+  m.def("gated_scan_record", [](int kind, int D, int V) { return k8s_gated_scan_record(kind, D, V); });
+  m.def("gated_scan", [](uintptr_t out, uintptr_t proj, long ld, int kind, int cq, int ck, int cv, int ci, int cf,
+                         int cg, uintptr_t fbias, uintptr_t ibias, uintptr_t lower, uintptr_t normw, uintptr_t state,
+                         uintptr_t cu_q, uintptr_t seq_slots, uintptr_t positions, int nseq, int H, int D, int V,
+                         float eps, float cap, int f32, int64_t s) {
+    check(k8s_gated_scan(P(out), P<float>(proj), ld, kind, cq, ck, cv, ci, cf, cg, P(fbias), P(ibias), P(lower),
+                         P(normw), P<float>(state), P<int>(cu_q), P<int>(seq_slots), P<int>(positions), nseq, H, D, V,
+                         eps, cap, f32, S(s)), "gated_scan");
   });
   m.def("moe_align", [](uintptr_t sorted_tok, uintptr_t pos, uintptr_t seg, uintptr_t tiles, int ntiles,
                         uintptr_t topk_idx, int P_, int top, int E, int BM, int64_t s) {

@@ -96,6 +96,15 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   return t;
 }
 
+// Workgroup barrier that waits for this wave's LDS traffic only: __syncthreads() also drains the outstanding global
+// loads, which would put the prefetched inputs of the next tokens back on the recurrence's latency chain.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0); vmcnt and expcnt untouched
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 // 32-bit mixing hash (murmur3 finalizer) used for counter-based RNG and deterministic init.
 __device__ __forceinline__ uint32_t fmix32(uint32_t h) {
   h ^= h >> 16; h *= 0x85ebca6bu; h ^= h >> 13; h *= 0xc2b2ae35u; h ^= h >> 16;

@@ -41,15 +41,6 @@ __global__ void shift_save_kernel(TA* __restrict__ state, const TA* __restrict__
   for (int i = threadIdx.x; i < W; i += blockDim.x) state[dst + i] = h[src + i];
 }
 
-// Workgroup barrier that waits for this wave's LDS traffic only: __syncthreads() also drains the outstanding global
-// loads, which would put the prefetched inputs of the next tokens back on the recurrence's latency chain.
-__device__ __forceinline__ void lds_barrier() {
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0); vmcnt and expcnt untouched
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-}
-
 // Chunk g of a varlen batch cut into chunks of Lc tokens per sequence: (sequence, chunk in the sequence, chunks of the
 // sequence), or sequence -1 when g is past the last chunk.  Idle (position < 0) and empty sequences have no chunks.
 struct WkvChunk { int s, c, n; };

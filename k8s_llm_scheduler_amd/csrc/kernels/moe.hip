@@ -1,27 +1,32 @@
-// Mixture of experts: softmax-top-k router, the sort of (token, choice) pairs by expert that feeds the grouped GEMMs
+// Mixture of experts: softmax- or sigmoid-top-k router, the sort of (token, choice) pairs by expert that feeds the grouped GEMMs
 // (stream32.hip gemm_any, `tiles` form), and the weighted combine with an optional gated shared expert.
 #include "common.h"
 
 namespace k8sllm {
 
-// One wave per token.  s = softmax(logits[t, :E]) in fp32; `top` rounds of arg-max (ties: the lowest index); weights
-// s_k / (sum of the chosen s + 1e-20) * scale.
+// One wave per token.  mode 0: s = softmax(logits[t, :E]) in fp32, weights s_k / (sum of the chosen s + 1e-20) * scale;
+// mode 1: s = sigmoid(logits), weights s_k * scale (not renormalised).  `top` rounds of arg-max (ties: the lowest index).
 __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ idx, float* __restrict__ w,
                                                        const float* __restrict__ logits, int ld, int E, int top,
-                                                       float scale) {
+                                                       float scale, int mode) {
   extern __shared__ float sc[];   // [E] scores, then [top] chosen scores
   const int t = blockIdx.x, lane = threadIdx.x;
   const float* z = logits + (size_t)t * ld;
-  float mx = -INFINITY;
-  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
-  mx = wave_max(mx);
-  float sum = 0.f;
-  for (int e = lane; e < E; e += 64) {
-    const float v = expf(z[e] - mx);
-    sc[e] = v;
-    sum += v;
+  float sum = 1.f;
+  if (mode == 1) {
+    for (int e = lane; e < E; e += 64) sc[e] = 1.f / (1.f + expf(-z[e]));
+  } else {
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+    mx = wave_max(mx);
+    sum = 0.f;
+    for (int e = lane; e < E; e += 64) {
+      const float v = expf(z[e] - mx);
+      sc[e] = v;
+      sum += v;
+    }
+    sum = wave_sum(sum);
   }
-  sum = wave_sum(sum);
   __syncthreads();
   float chosen_sum = 0.f;
   for (int k = 0; k < top; ++k) {
@@ -52,7 +57,8 @@ __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ idx, fl
     }
     __syncthreads();
   }
-  for (int k = lane; k < top; k += 64) w[(size_t)t * top + k] = sc[E + k] / (chosen_sum + 1e-20f) * scale;
+  const float norm = mode == 1 ? 1.f : 1.f / (chosen_sum + 1e-20f);
+  for (int k = lane; k < top; k += 64) w[(size_t)t * top + k] = sc[E + k] * norm * scale;
 }
 
 // One workgroup.  Pairs p = t * top + k are sorted by expert (any order inside an expert: rows are independent):
@@ -104,7 +110,8 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(int* __restrict__ sorte
   }
 }
 
-// z[t] = sum_k w[t, k] D[pos[t, k]] + gate_t * shared[t], gate_t = sigmoid(logits[t, sg_col]) (sg_col < 0: 1).
+// z[t] = sum_k w[t, k] D[pos[t, k]] + gate_t * shared[t], gate_t = sigmoid(logits[t, sg_col]) (sg_col < 0: 1);
+// w == null: plain sum (experts whose weight was applied to their input).
 template <typename TA>
 __global__ void moe_combine_kernel(TA* __restrict__ z, const TA* __restrict__ D, const int* __restrict__ pos,
                                    const float* __restrict__ w, const TA* __restrict__ shared,
@@ -115,7 +122,7 @@ __global__ void moe_combine_kernel(TA* __restrict__ z, const TA* __restrict__ D,
   for (int i = threadIdx.x; i < W; i += blockDim.x) {
     float a = 0.f;
     for (int k = 0; k < top; ++k)
-      a = fmaf(w[(size_t)t * top + k], ldf(D, (size_t)pos[(size_t)t * top + k] * W + i), a);
+      a = fmaf(w != nullptr ? w[(size_t)t * top + k] : 1.f, ldf(D, (size_t)pos[(size_t)t * top + k] * W + i), a);
     if (shared != nullptr) a = fmaf(gate, ldf(shared, (size_t)t * W + i), a);
     stf(z, (size_t)t * W + i, a);
   }
@@ -126,10 +133,10 @@ __global__ void moe_combine_kernel(TA* __restrict__ z, const TA* __restrict__ D,
 using namespace k8sllm;
 
 extern "C" int k8s_moe_route(int* idx, float* w, const float* logits, int ld, int T, int E, int top, float scale,
-                             hipStream_t s) {
+                             int mode, hipStream_t s) {
   if (T <= 0) return 0;
-  if (E <= 0 || top <= 0 || top > E || E > 8192) return -1;
-  moe_route_kernel<<<T, 64, (size_t)(E + top) * sizeof(float), s>>>(idx, w, logits, ld, E, top, scale);
+  if (E <= 0 || top <= 0 || top > E || E > 8192 || mode < 0 || mode > 1) return -1;
+  moe_route_kernel<<<T, 64, (size_t)(E + top) * sizeof(float), s>>>(idx, w, logits, ld, E, top, scale, mode);
   return (int)hipGetLastError();
 }
 

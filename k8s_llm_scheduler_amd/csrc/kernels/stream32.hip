@@ -7,23 +7,23 @@
 
 namespace k8sllm {
 
-// out[t, :] = float(table[ids[t], :])
+// out[t, :] = float(table[ids[t], :]) * scale
 template <typename TA>
 __global__ void embed_rows_kernel(float* __restrict__ out, const int* __restrict__ ids, const TA* __restrict__ table,
-                                  int W, int vocab) {
+                                  int W, int vocab, float scale) {
   const int t = blockIdx.x;
   int id = ids[t];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
-  for (int i = threadIdx.x; i < W; i += blockDim.x) out[(size_t)t * W + i] = ldf(table, (size_t)id * W + i);
+  for (int i = threadIdx.x; i < W; i += blockDim.x) out[(size_t)t * W + i] = ldf(table, (size_t)id * W + i) * scale;
 }
 
 // x[t] += mult * branch[t] + rowvec (each optional), stored back in fp32; then (w != null)
-// out[t] = x[t] / sqrt(mean(x[t]^2) + eps) * (offset + w).  One workgroup per row; the row stays in registers / LDS
-// between the add and the norm.
+// out[t] = x[t] / sqrt(mean(x[t]^2) + eps) * (offset + w), the mean taken over each of `groups` equal consecutive parts
+// of the row by itself.  One workgroup per row; groups > 1: one wave per part.
 template <typename TA>
 __global__ __launch_bounds__(256) void resnorm_kernel(float* __restrict__ x, const TA* __restrict__ branch, float mult,
                                                       const TA* __restrict__ rowvec, const TA* __restrict__ w,
-                                                      float offset, float eps, TA* __restrict__ out, int W) {
+                                                      float offset, float eps, TA* __restrict__ out, int W, int groups) {
   __shared__ float red[16];
   const size_t base = (size_t)blockIdx.x * W;
   float ss = 0.f;
@@ -36,24 +36,45 @@ __global__ __launch_bounds__(256) void resnorm_kernel(float* __restrict__ x, con
     ss += v * v;
   }
   if (w == nullptr) return;
-  ss = block_sum(ss, red);
-  const float inv = 1.0f / sqrtf(ss / (float)W + eps);
-  for (int i = threadIdx.x; i < W; i += blockDim.x)
-    stf(out, base + i, x[base + i] * inv * (offset + ldf(w, i)));
+  if (groups <= 1) {
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)W + eps);
+    for (int i = threadIdx.x; i < W; i += blockDim.x)
+      stf(out, base + i, x[base + i] * inv * (offset + ldf(w, i)));
+    return;
+  }
+  __syncthreads();   // the updated row is read back by other threads
+  const int Wg = W / groups, wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+  for (int g = wave; g < groups; g += nw) {
+    const size_t b = base + (size_t)g * Wg;
+    float sg = 0.f;
+    for (int i = lane; i < Wg; i += 64) {
+      const float v = x[b + i];
+      sg += v * v;
+    }
+    sg = wave_sum(sg);
+    const float inv = 1.0f / sqrtf(sg / (float)Wg + eps);
+    for (int i = lane; i < Wg; i += 64) stf(out, b + i, x[b + i] * inv * (offset + ldf(w, (size_t)g * Wg + i)));
+  }
 }
 
 // kinds: 0 gelu_tanh(g) * u, 1 g' * sigmoid(alpha g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, +-limit)
-// (limit <= 0: no clamp) -- both read [T, 2F] = [gate | up]; 2 tanh, 3 silu: elementwise on [T, F].
+// (limit <= 0: no clamp) -- both read [T, 2F] = [gate | up]; 2 tanh, 3 silu, 4 erf-gelu: elementwise on [T, F].
+// Elementwise kinds take a factor per row: logical row i is row row_map[i] (or i) and its input is multiplied by
+// row_scale[i] before the function (experts whose router weight scales their input).
 template <typename TA>
 __global__ void act_kernel(TA* __restrict__ out, const TA* __restrict__ x, int T, int F, int kind, float limit,
-                           float alpha) {
+                           float alpha, const float* __restrict__ row_scale, const int* __restrict__ row_map) {
   const size_t n = (size_t)T * F;
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
     const size_t t = i / F, c = i - t * F;
     float y;
+    size_t o = i;
     if (kind >= 2) {
-      const float v = ldf(x, i);
-      y = kind == 2 ? tanhf(v) : v / (1.f + expf(-v));
+      if (row_map != nullptr) o = (size_t)row_map[t] * F + c;
+      float v = ldf(x, o);
+      if (row_scale != nullptr) v *= row_scale[t];
+      y = kind == 2 ? tanhf(v) : kind == 3 ? v / (1.f + expf(-v)) : 0.5f * v * (1.f + erff(v * 0.7071067811865476f));
     } else {
       float g = ldf(x, t * 2 * F + c), u = ldf(x, t * 2 * F + F + c);
       if (kind == 0) {
@@ -66,7 +87,7 @@ __global__ void act_kernel(TA* __restrict__ out, const TA* __restrict__ x, int T
         y = g / (1.f + expf(-alpha * g)) * (u + 1.f);
       }
     }
-    stf(out, i, y);
+    stf(out, o, y);
   }
 }
 
@@ -244,36 +265,38 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(TO* __restrict__ C, cons
 
 using namespace k8sllm;
 
-extern "C" int k8s_embed_rows(float* out, const int* ids, const void* table, int T, int W, int vocab, int f32,
-                              hipStream_t s) {
+extern "C" int k8s_embed_rows(float* out, const int* ids, const void* table, int T, int W, int vocab, float scale,
+                              int f32, hipStream_t s) {
   if (T <= 0) return 0;
   if (W <= 0 || vocab <= 0) return -1;
-  if (f32) embed_rows_kernel<float><<<T, 256, 0, s>>>(out, ids, (const float*)table, W, vocab);
-  else embed_rows_kernel<bf16_t><<<T, 256, 0, s>>>(out, ids, (const bf16_t*)table, W, vocab);
+  if (f32) embed_rows_kernel<float><<<T, 256, 0, s>>>(out, ids, (const float*)table, W, vocab, scale);
+  else embed_rows_kernel<bf16_t><<<T, 256, 0, s>>>(out, ids, (const bf16_t*)table, W, vocab, scale);
   return (int)hipGetLastError();
 }
 
 extern "C" int k8s_resnorm(float* x, const void* branch, float mult, const void* rowvec, const void* w, float offset,
-                           float eps, void* out, int T, int W, int f32, hipStream_t s) {
+                           float eps, void* out, int T, int W, int groups, int f32, hipStream_t s) {
   if (T <= 0) return 0;
-  if (W <= 0 || (w != nullptr && out == nullptr)) return -1;
+  if (W <= 0 || (w != nullptr && out == nullptr) || groups < 1 || W % groups) return -1;
   if (f32)
     resnorm_kernel<float><<<T, 256, 0, s>>>(x, (const float*)branch, mult, (const float*)rowvec, (const float*)w,
-                                            offset, eps, (float*)out, W);
+                                            offset, eps, (float*)out, W, groups);
   else
     resnorm_kernel<bf16_t><<<T, 256, 0, s>>>(x, (const bf16_t*)branch, mult, (const bf16_t*)rowvec, (const bf16_t*)w,
-                                             offset, eps, (bf16_t*)out, W);
+                                             offset, eps, (bf16_t*)out, W, groups);
   return (int)hipGetLastError();
 }
 
-extern "C" int k8s_act(void* out, const void* x, int T, int F, int kind, float limit, float alpha, int f32,
-                       hipStream_t s) {
+extern "C" int k8s_act(void* out, const void* x, int T, int F, int kind, float limit, float alpha,
+                       const float* row_scale, const int* row_map, int f32, hipStream_t s) {
   if (T <= 0 || F <= 0) return 0;
-  if (kind < 0 || kind > 3) return -1;
+  if (kind < 0 || kind > 4 || (kind < 2 && (row_scale != nullptr || row_map != nullptr))) return -1;
   const size_t n = (size_t)T * F;
   const int blocks = (int)((n + 255) / 256 > 4096 ? 4096 : (n + 255) / 256);
-  if (f32) act_kernel<float><<<blocks, 256, 0, s>>>((float*)out, (const float*)x, T, F, kind, limit, alpha);
-  else act_kernel<bf16_t><<<blocks, 256, 0, s>>>((bf16_t*)out, (const bf16_t*)x, T, F, kind, limit, alpha);
+  if (f32) act_kernel<float><<<blocks, 256, 0, s>>>((float*)out, (const float*)x, T, F, kind, limit, alpha,
+                                                    row_scale, row_map);
+  else act_kernel<bf16_t><<<blocks, 256, 0, s>>>((bf16_t*)out, (const bf16_t*)x, T, F, kind, limit, alpha,
+                                                row_scale, row_map);
   return (int)hipGetLastError();
 }
 

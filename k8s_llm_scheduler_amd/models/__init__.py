@@ -15,18 +15,21 @@ def _architecture(c: dict) -> str:
 
 def load_config(name_or_path: str):
     """The configuration object of a preset or checkpoint."""
-    from . import putulorn
+    from . import putulorn, rupatar
     from .config import get_config
 
-    if name_or_path in putulorn.PRESETS:
-        return putulorn.PRESETS[name_or_path]
+    designs = (putulorn, rupatar)
+    for d in designs:
+        if name_or_path in d.PRESETS:
+            return d.PRESETS[name_or_path]
     p = Path(name_or_path)
     if p.is_dir():
         p = p / "config.json"
     if p.is_file():
         c = json.loads(p.read_text())
-        if _architecture(c) == putulorn.ARCHITECTURE:
-            return putulorn.config_from_json(c, p.parent.name or "putulorn")
+        for d in designs:
+            if _architecture(c) == d.ARCHITECTURE:
+                return d.config_from_json(c, p.parent.name or d.ARCHITECTURE.lower())
     return get_config(name_or_path)
 
 
@@ -35,9 +38,12 @@ def model_class(cfg):
     from .config import LlamaConfig
     from .llama import LlamaModel
     from .putulorn import PutulornConfig, PutulornModel
+    from .rupatar import RupatarConfig, RupatarModel
 
     if isinstance(cfg, PutulornConfig):
         return PutulornModel
+    if isinstance(cfg, RupatarConfig):
+        return RupatarModel
     if isinstance(cfg, LlamaConfig):
         return LlamaModel
     raise TypeError(f"no model class for {type(cfg).__name__}")

@@ -64,8 +64,11 @@ def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float,
 
 
 def rope_table(head_dim: int, max_pos: int, theta: float, scaling: Optional[dict] = None) -> torch.Tensor:
-    """[max_pos, head_dim] fp32: cos in [:, :D/2], sin in [:, D/2:] (llama3 scaling if given)."""
+    """[max_pos, head_dim] fp32: cos in [:, :D/2], sin in [:, D/2:] (llama3 or linear scaling if given; linear:
+    every frequency divided by ``factor``).  Angles are formed in float64."""
     inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float64) / head_dim))
+    if scaling and scaling.get("rope_type", scaling.get("type")) == "linear":
+        inv = inv / float(scaling["factor"])
     if scaling and scaling.get("rope_type", scaling.get("type")) == "llama3":
         factor = scaling["factor"]
         lo, hi = scaling["low_freq_factor"], scaling["high_freq_factor"]
@@ -483,30 +486,41 @@ def write_token_stop(s: int, tok: int, tokens, ctx_inc, hist, steps, stop) -> No
 
 
 # ----------------------------------------------------------------------------- fp32 residual stream, gated activations
-ACT_GELU_TANH, ACT_SWISH_CLAMP, ACT_TANH, ACT_SILU = 0, 1, 2, 3
+ACT_GELU_TANH, ACT_SWISH_CLAMP, ACT_TANH, ACT_SILU, ACT_GELU_ERF = 0, 1, 2, 3, 4
 
 
-def embed_rows(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
-    """fp32 rows of the embedding table (the residual stream starts in fp32)."""
-    return table.index_select(0, ids.long()).float()
+def embed_rows(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """fp32 rows of the embedding table times ``scale`` (the residual stream starts in fp32)."""
+    return table.index_select(0, ids.long()).float() * scale
 
 
-def resnorm(x: torch.Tensor, branch, mult: float, rowvec, w, offset: float, eps: float, out_dtype):
-    """x (fp32, in place) += mult * branch + rowvec; returns x / sqrt(mean(x^2) + eps) * (offset + w) or None."""
+def resnorm(x: torch.Tensor, branch, mult: float, rowvec, w, offset: float, eps: float, out_dtype, groups: int = 1):
+    """x (fp32, in place) += mult * branch + rowvec; returns x / sqrt(mean(x^2) + eps) * (offset + w) or None, the
+    mean taken over each of ``groups`` equal consecutive parts of a row by itself."""
     if branch is not None:
         x.add_(branch.float() * mult)
     if rowvec is not None:
         x.add_(rowvec.float())
     if w is None:
         return None
-    y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * (offset + w.float())
+    T, W = x.shape
+    xg = x.view(T, groups, W // groups)
+    y = (xg * torch.rsqrt(xg.pow(2).mean(-1, keepdim=True) + eps)).reshape(T, W) * (offset + w.float())
     return y.to(out_dtype)
 
 
-def act(x: torch.Tensor, kind: int, limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
-    """Gated kinds take [T, 2F] = [gate | up] and return [T, F]; ACT_TANH / ACT_SILU are elementwise."""
-    if kind in (ACT_TANH, ACT_SILU):
+def act(x: torch.Tensor, kind: int, limit: float = 0.0, alpha: float = 1.0, row_scale=None, row_map=None) -> torch.Tensor:
+    """Gated kinds take [T, 2F] = [gate | up] and return [T, F]; ACT_TANH / ACT_SILU / ACT_GELU_ERF are elementwise and
+    take a factor per row: logical row i is row ``row_map[i]`` (or i), its input times ``row_scale[i]``."""
+    if kind in (ACT_TANH, ACT_SILU, ACT_GELU_ERF):
         f = x.float()
+        if row_scale is not None:
+            sc = row_scale.float()
+            if row_map is not None:
+                sc = torch.zeros(x.shape[0]).index_copy_(0, row_map.long(), sc)
+            f = f * sc.unsqueeze(-1)
+        if kind == ACT_GELU_ERF:
+            return (0.5 * f * (1.0 + torch.erf(f / math.sqrt(2.0)))).to(x.dtype)
         return (torch.tanh(f) if kind == ACT_TANH else f * torch.sigmoid(f)).to(x.dtype)
     F = x.shape[-1] // 2
     g, u = x[..., :F].float(), x[..., F:].float()
@@ -638,12 +652,16 @@ def latent_attention(q_abs, q, cache, block_tables, tok_seq, positions, C: int, 
 
 
 # ----------------------------------------------------------------------------- mixture of experts
-def moe_route(logits: torch.Tensor, E: int, top: int, scale: float):
-    """softmax over the first E columns, the ``top`` largest (ties: lowest index), weights s / (sum s + 1e-20) * scale."""
-    s = torch.softmax(logits[:, :E].float(), -1)
+def moe_route(logits: torch.Tensor, E: int, top: int, scale: float, score: str = "softmax"):
+    """Scores over the first E columns, the ``top`` largest (ties: lowest index).  "softmax": weights
+    s / (sum of the chosen s + 1e-20) * scale; "sigmoid": weights s * scale, not renormalised."""
+    z = logits[:, :E].float()
+    s = torch.sigmoid(z) if score == "sigmoid" else torch.softmax(z, -1)
     w, idx = torch.sort(s, dim=-1, descending=True, stable=True)
     w, idx = w[:, :top], idx[:, :top]
-    return idx.int().contiguous(), (w / (w.sum(-1, keepdim=True) + 1e-20) * scale).contiguous()
+    if score != "sigmoid":
+        w = w / (w.sum(-1, keepdim=True) + 1e-20)
+    return idx.int().contiguous(), (w * scale).contiguous()
 
 
 def moe_align(topk_idx: torch.Tensor, E: int, BM: int):
@@ -667,11 +685,179 @@ def moe_align(topk_idx: torch.Tensor, E: int, BM: int):
     return (order // top).int(), pos.int(), seg, tiles
 
 
-def moe_combine(D, pos_of_pair, topk_w, shared, logits, sg_col: int, out_dtype):
-    """z[t] = sum_k w[t, k] D[pos[t, k]] + sigmoid(logits[t, sg_col]) * shared[t]."""
-    T, top = topk_w.shape
-    z = (D.float()[pos_of_pair.long().view(T, top)] * topk_w.unsqueeze(-1)).sum(1)
+def moe_combine(D, pos_of_pair, topk_w, shared, logits, sg_col: int, out_dtype, top: int = 0):
+    """z[t] = sum_k w[t, k] D[pos[t, k]] + sigmoid(logits[t, sg_col]) * shared[t]  (topk_w None: plain sum)."""
+    top = topk_w.shape[1] if topk_w is not None else top
+    T = pos_of_pair.numel() // top
+    rows = D.float()[pos_of_pair.long().view(T, top)]
+    z = (rows * topk_w.unsqueeze(-1) if topk_w is not None else rows).sum(1)
     if shared is not None:
         gate = torch.sigmoid(logits[:, sg_col].float()).unsqueeze(-1) if sg_col >= 0 else 1.0
         z = z + gate * shared.float()
     return z.to(out_dtype)
+
+
+# ----------------------------------------------------------------------------- windowed attention with pooled blocks
+def pool_entry(bt_row, b: int, P: int, bs: int) -> int:
+    """Entry of pooled block b: it lives with the page that holds its first token; a page has ceil(bs / P) entries."""
+    ppb = -(-bs // P)
+    page = b * P // bs
+    first = -(-(page * bs) // P)
+    return int(bt_row[page]) * ppb + (b - first)
+
+
+def window_kv_write(kcache, vcache, qkv, koff: int, voff: int, qb, kb, vb, cos_sin, positions, slot_mapping, vfirst_in,
+                    vfirst_out, lam: float, H: int, G: int, D: int, V: int, dims: int, eps: float, unit: bool) -> None:
+    """Per token: q (first H D columns of qkv, rewritten in place) and k (at koff) get their bias, the rotation of the
+    pairs (2i, 2i + 1), i < dims / 2, by cos_sin[pos] = [cos | sin], and (``unit``) x / sqrt(mean(x^2) + eps) per head;
+    v (at voff) gets its bias and (``vfirst_in``) becomes (1 - lam) v + lam vfirst_in; ``vfirst_out`` receives v in
+    fp32.  k, v go to kcache [slots, G, D] / vcache [slots, G, V] at the tokens' slots (negative: not written); rows
+    with a negative position are skipped."""
+    T = qkv.shape[0]
+    live = positions >= 0
+    half = dims // 2
+    cs = cos_sin[positions.long().clamp(min=0)] if dims else None
+
+    def prep(x, bias, n):
+        x = x.float().view(T, n, D)
+        if bias is not None:
+            x = x + bias.float().view(n, D)
+        if dims:
+            c, s = cs[:, None, :half], cs[:, None, half:]
+            a, b = x[..., 0:dims:2], x[..., 1:dims:2]
+            x = x.clone()
+            x[..., 0:dims:2], x[..., 1:dims:2] = a * c - b * s, b * c + a * s
+        if unit:
+            x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+        return x
+
+    q = prep(qkv[:, :H * D], qb, H).reshape(T, H * D)
+    k = prep(qkv[:, koff:koff + G * D], kb, G)
+    v = qkv[:, voff:voff + G * V].float()
+    if vb is not None:
+        v = v + vb.float()
+    if vfirst_in is not None:
+        v = (1.0 - lam) * v + lam * vfirst_in
+    if vfirst_out is not None:
+        vfirst_out[live] = v[live]
+    qkv[live, :H * D] = q[live].to(qkv.dtype)
+    ok = live & (slot_mapping >= 0)
+    kcache[slot_mapping[ok].long()] = k[ok].to(kcache.dtype)
+    vcache[slot_mapping[ok].long()] = v[ok].view(-1, G, V).to(vcache.dtype)
+
+
+def window_pool(kpool, vpool, kcache, vcache, block_tables, tok_seq, positions, P: int, bs: int) -> None:
+    """For every token that ends a block of P tokens: the fp32 mean of the block's cached keys / values."""
+    for t in range(positions.shape[0]):
+        p = int(positions[t])
+        if p < 0 or (p + 1) % P:
+            continue
+        b = p // P
+        bt = block_tables[int(tok_seq[t])].long()
+        js = torch.arange(b * P, b * P + P)
+        slots = bt[js // bs] * bs + js % bs
+        e = pool_entry(bt, b, P, bs)
+        kpool[e] = kcache[slots].float().mean(0)
+        vpool[e] = vcache[slots].float().mean(0)
+
+
+def window_attention(q, gate, kcache, vcache, kpool, vpool, block_tables, tok_seq, positions, H: int, G: int, D: int,
+                     V: int, window: int, P: int, scale: float, sink: bool, bs: int, out_dtype):
+    """Token t at position p attends the cached tokens max(0, p - window + 1) .. p (window <= 0: all) and the pooled
+    blocks b with b P + P - 1 <= p - window, in one softmax (``sink``: one more unit in the denominator); query head h
+    uses key / value head h // (H / G).  The result times sigmoid(gate) if given.  [T, H V]."""
+    T = q.shape[0]
+    out = torch.zeros(T, H, V)
+    qf = q.float().reshape(T, -1)[:, :H * D].view(T, H, D)
+    R = H // G
+    for t in range(T):
+        p = int(positions[t])
+        if p < 0:
+            continue
+        lo = 0 if window <= 0 else max(0, p - window + 1)
+        nb = (p - window + 1) // P if (window > 0 and P > 0 and p - window + 1 >= P) else 0
+        bt = block_tables[int(tok_seq[t])].long()
+        js = torch.arange(lo, p + 1)
+        slots = bt[js // bs] * bs + js % bs
+        K, Vv = kcache[slots].float(), vcache[slots].float()
+        if nb:
+            es = torch.tensor([pool_entry(bt, b, P, bs) for b in range(nb)])
+            K, Vv = torch.cat([kpool[es], K]), torch.cat([vpool[es], Vv])
+        for h in range(H):
+            g = h // R
+            s = (K[:, g] @ qf[t, h]) * scale
+            mx = s.max().clamp(min=0.0) if sink else s.max()
+            e = torch.exp(s - mx)
+            den = e.sum() + (torch.exp(-mx) if sink else 0.0)
+            out[t, h] = (e / den) @ Vv[:, g]
+    out = out.reshape(T, H * V)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float())
+    return out.to(out_dtype)
+
+
+# ----------------------------------------------------------------------------- gated matrix-state recurrences
+SCAN_HGRN2, SCAN_MLSTM = 0, 1
+
+
+def gated_scan_record(kind: int, D: int, V: int) -> int:
+    return D * V + (D + 1 if kind == SCAN_MLSTM else 0)
+
+
+def gated_scan(proj, kind: int, cols: dict, fbias, ibias, lower, normw, state, cu_q, seq_slots, positions, H: int,
+               D: int, V: int, eps: float, cap: float, out_dtype):
+    """``proj`` fp32 [T, ld] holds the parts at the column offsets ``cols``; ``state`` [slots, H, record] fp32.
+    SCAN_HGRN2: f = low + (1 - low) sigmoid(zf + bf), S <- diag(f) S + (1 - f) v^T, o = S^T silu(zq),
+    y = o / rms(o) * normw [V].  SCAN_MLSTM: i = cap tanh((zi + bi) / cap), f = logsigmoid(cap tanh((zf + bf) / cap)),
+    m' = max(f + m, i), S <- e^(f + m - m') S + e^(i - m') k v^T, n likewise, o = S^T q / (max(|n . q|, e^(-m')) + 1e-6)
+    with q = zq / sqrt(D), y = o / rms(o) * normw [H V] * sigmoid(zg).  A portion at position 0 starts from zero."""
+    T = proj.shape[0]
+    pf = proj.float()
+    out = torch.zeros(T, H, V)
+    cu = cu_q.tolist()
+    part = lambda key, n: pf[:, cols[key]:cols[key] + H * n].view(T, H, n)
+    v = part("v", V)
+    if kind == SCAN_HGRN2:
+        zq = part("q", D)
+        q = zq * torch.sigmoid(zq)
+        low = lower.float().view(H, D)
+        zf = part("f", D) + (fbias.float().view(H, D) if fbias is not None else 0.0)
+        f = low + (1.0 - low) * torch.sigmoid(zf)
+    else:
+        q = part("q", D) / math.sqrt(D)
+        k = part("k", D)
+        zi = pf[:, cols["i"]:cols["i"] + H] + (ibias.float() if ibias is not None else 0.0)
+        zf = pf[:, cols["f"]:cols["f"] + H] + (fbias.float() if fbias is not None else 0.0)
+        ig = cap * torch.tanh(zi / cap)
+        fg = torch.nn.functional.logsigmoid(cap * torch.tanh(zf / cap))
+    for s in range(len(cu) - 1):
+        a, b = cu[s], cu[s + 1]
+        if b <= a or int(positions[a]) < 0:
+            continue
+        slot = int(seq_slots[s])
+        rec = torch.zeros(H, gated_scan_record(kind, D, V)) if int(positions[a]) == 0 else state[slot].clone()
+        S = rec[:, :D * V].reshape(H, D, V).clone()
+        if kind == SCAN_MLSTM:
+            n, m = rec[:, D * V:D * V + D].clone(), rec[:, D * V + D].clone()
+        for t in range(a, b):
+            if kind == SCAN_HGRN2:
+                S = f[t].unsqueeze(2) * S + (1.0 - f[t]).unsqueeze(2) * v[t].unsqueeze(1)
+                o = torch.einsum("hdv,hd->hv", S, q[t])
+            else:
+                mn = torch.maximum(fg[t] + m, ig[t])
+                ka, kb = torch.exp(fg[t] + m - mn), torch.exp(ig[t] - mn)
+                m = mn
+                S = ka[:, None, None] * S + kb[:, None, None] * k[t].unsqueeze(2) * v[t].unsqueeze(1)
+                n = ka[:, None] * n + kb[:, None] * k[t]
+                den = torch.maximum((n * q[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
+                o = torch.einsum("hdv,hd->hv", S, q[t]) / den[:, None]
+            out[t] = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+        state[slot, :, :D * V] = S.reshape(H, D * V)
+        if kind == SCAN_MLSTM:
+            state[slot, :, D * V:D * V + D] = n
+            state[slot, :, D * V + D] = m
+    if kind == SCAN_HGRN2:
+        y = (out * normw.float().view(1, 1, V)).reshape(T, H * V)
+    else:
+        y = out.reshape(T, H * V) * normw.float() * torch.sigmoid(pf[:, cols["g"]:cols["g"] + H * V])
+    return y.to(out_dtype)

@@ -1,7 +1,7 @@
-"""Ops of models with an fp32 residual stream, recurrent / latent-attention mixers and mixtures of experts.
+"""Ops of models with an fp32 residual stream, recurrent / windowed- or latent-attention mixers and mixtures of experts.
 
 Same dispatch rule as the rest of :mod:`..ops`: CUDA (= HIP) tensors always run the gfx950 kernels
-(``stream32.hip``, ``mixers.hip``, ``moe.hip``) and raise when the extension is missing; CPU tensors run the fp32
+(``stream32.hip``, ``mixers.hip``, ``window_attn.hip``, ``gated_scan.hip``, ``moe.hip``) and raise when the extension is missing; CPU tensors run the fp32
 reference in :mod:`.reference` (the CPU test-suite).  Every op takes bf16 or true-fp32 activations / weights (the
 ``f32`` flag of the kernels); what a design computes in fp32 regardless (residual sum, recurrent state, decays, router,
 attention scores) is fp32 in both.
@@ -15,7 +15,8 @@ from typing import Optional
 import torch
 
 from . import reference as ref
-from .reference import ACT_GELU_TANH, ACT_SILU, ACT_SWISH_CLAMP, ACT_TANH  # noqa: F401
+from .reference import ACT_GELU_ERF, ACT_GELU_TANH, ACT_SILU, ACT_SWISH_CLAMP, ACT_TANH  # noqa: F401
+from .reference import SCAN_HGRN2, SCAN_MLSTM  # noqa: F401
 
 BF16, F32, I32 = torch.bfloat16, torch.float32, torch.int32
 GROUP_BM = 64   # row-tile height of the grouped GEMM (gemm_any_kernel's BM)
@@ -53,44 +54,58 @@ def _f32(dtype) -> int:
 
 
 # ----------------------------------------------------------------------------- residual stream
-def embed_rows(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
-    """fp32 [T, W] rows of ``table`` (bf16 or fp32)."""
+def embed_rows(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """fp32 [T, W] rows of ``table`` (bf16 or fp32) times ``scale``."""
     if not _gpu(ids, table):
-        return ref.embed_rows(ids, table)
+        return ref.embed_rows(ids, table, scale)
     T, W = ids.shape[0], table.shape[1]
     out = torch.empty(T, W, dtype=F32, device=table.device)
-    _native().embed_rows(out.data_ptr(), _p(ids, I32, "ids"), _p(table), T, W, table.shape[0], _f32(table.dtype), -1)
+    _native().embed_rows(out.data_ptr(), _p(ids, I32, "ids"), _p(table), T, W, table.shape[0], float(scale),
+                         _f32(table.dtype), -1)
     return out
 
 
 def resnorm(x: torch.Tensor, w: Optional[torch.Tensor], eps: float, *, branch: Optional[torch.Tensor] = None,
             mult: float = 1.0, rowvec: Optional[torch.Tensor] = None, offset: float = 0.0,
-            out_dtype=BF16) -> Optional[torch.Tensor]:
+            out_dtype=BF16, groups: int = 1) -> Optional[torch.Tensor]:
     """``x`` (fp32 [T, W], updated in place) += mult * branch + rowvec; returns rms-norm(x) * (offset + w) in
-    ``out_dtype``, or None when ``w`` is None (add only)."""
+    ``out_dtype``, or None when ``w`` is None (add only).  ``groups`` > 1: every one of that many equal consecutive
+    parts of a row is divided by its own root mean square."""
     if x.dtype != F32:
         raise TypeError("the residual stream is fp32")
-    if not _gpu(x, w, branch, rowvec):
-        return ref.resnorm(x, branch, mult, rowvec, w, offset, eps, out_dtype)
     T, W = x.shape
+    if groups < 1 or W % groups:
+        raise ValueError(f"resnorm: {groups} groups do not divide the width {W}")
+    if not _gpu(x, w, branch, rowvec):
+        return ref.resnorm(x, branch, mult, rowvec, w, offset, eps, out_dtype, groups)
     out = torch.empty(T, W, dtype=out_dtype, device=x.device) if w is not None else None
     f32 = _f32(out_dtype)
     for t, n in ((branch, "branch"), (rowvec, "rowvec"), (w, "w")):
         if t is not None and t.dtype != out_dtype:
             raise TypeError(f"{n}: expected {out_dtype}, got {t.dtype}")
     _native().resnorm(_p(x), _p(branch), float(mult), _p(rowvec), _p(w), float(offset), float(eps), _p(out), T, W,
-                      f32, -1)
+                      int(groups), f32, -1)
     return out
 
 
-def act(x: torch.Tensor, kind: int, limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
-    """Gated kinds (ACT_GELU_TANH, ACT_SWISH_CLAMP): [T, 2F] = [gate | up] -> [T, F]; ACT_TANH / ACT_SILU: elementwise."""
-    if not _gpu(x):
-        return ref.act(x, kind, limit, alpha)
+def act(x: torch.Tensor, kind: int, limit: float = 0.0, alpha: float = 1.0, *,
+        row_scale: Optional[torch.Tensor] = None, row_map: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Gated kinds (ACT_GELU_TANH, ACT_SWISH_CLAMP): [T, 2F] = [gate | up] -> [T, F]; ACT_TANH / ACT_SILU / ACT_GELU_ERF
+    (exact gelu): elementwise.  Elementwise kinds take an fp32 factor per row, ``row_scale`` [T]: logical row i is row
+    ``row_map[i]`` (a permutation; default i) and its input is multiplied by ``row_scale[i]`` before the function."""
+    gated = kind in (ACT_GELU_TANH, ACT_SWISH_CLAMP)
+    if gated and (row_scale is not None or row_map is not None):
+        raise ValueError("act: row factors go with the elementwise kinds")
+    if not _gpu(x, row_scale, row_map):
+        return ref.act(x, kind, limit, alpha, row_scale, row_map)
     T = x.shape[0]
-    F = x.shape[1] // 2 if kind in (ACT_GELU_TANH, ACT_SWISH_CLAMP) else x.shape[1]
+    F = x.shape[1] // 2 if gated else x.shape[1]
+    for t, n in ((row_scale, "row_scale"), (row_map, "row_map")):
+        if t is not None and t.numel() != T:
+            raise ValueError(f"act: {n} must have one entry per row")
     out = torch.empty(T, F, dtype=x.dtype, device=x.device)
-    _native().act(out.data_ptr(), _p(x), T, F, kind, float(limit or 0.0), float(alpha), _f32(x.dtype), -1)
+    _native().act(out.data_ptr(), _p(x), T, F, kind, float(limit or 0.0), float(alpha), _p(row_scale, F32, "row_scale"),
+                  _p(row_map, I32, "row_map"), _f32(x.dtype), -1)
     return out
 
 
@@ -303,16 +318,20 @@ def latent_attention(q_abs: torch.Tensor, q: torch.Tensor, cache: torch.Tensor, 
 
 
 # ----------------------------------------------------------------------------- mixture of experts
-def moe_route(logits: torch.Tensor, E: int, top: int, scale: float):
-    """fp32 router logits [T, >= E] -> (expert ids int32 [T, top], weights fp32 [T, top])."""
+def moe_route(logits: torch.Tensor, E: int, top: int, scale: float, score: str = "softmax"):
+    """fp32 router logits [T, >= E] -> (expert ids int32 [T, top], weights fp32 [T, top]).  ``score``: "softmax"
+    (weights renormalised over the chosen experts) or "sigmoid" (the chosen experts' scores as they are)."""
     if logits.dtype != F32:
         raise TypeError("router logits are fp32")
+    if score not in ("softmax", "sigmoid"):
+        raise ValueError(f"moe_route: unknown score {score!r}")
     if not _gpu(logits):
-        return ref.moe_route(logits, E, top, scale)
+        return ref.moe_route(logits, E, top, scale, score)
     T = logits.shape[0]
     idx = torch.empty(T, top, dtype=I32, device=logits.device)
     w = torch.empty(T, top, dtype=F32, device=logits.device)
-    _native().moe_route(idx.data_ptr(), w.data_ptr(), _p(logits), logits.stride(0), T, E, top, float(scale), -1)
+    _native().moe_route(idx.data_ptr(), w.data_ptr(), _p(logits), logits.stride(0), T, E, top, float(scale),
+                        int(score == "sigmoid"), -1)
     return idx, w
 
 
@@ -333,14 +352,151 @@ def moe_align(topk_idx: torch.Tensor, E: int):
     return sorted_tok, pos, seg, tiles
 
 
-def moe_combine(D: torch.Tensor, pos_of_pair: torch.Tensor, topk_w: torch.Tensor, shared: Optional[torch.Tensor],
-                logits: torch.Tensor, sg_col: int) -> torch.Tensor:
-    """z[t] = sum_k w[t, k] D[pos[t, k]] + sigmoid(logits[t, sg_col]) * shared[t]  (sg_col < 0: ungated)."""
+def moe_combine(D: torch.Tensor, pos_of_pair: torch.Tensor, topk_w: Optional[torch.Tensor],
+                shared: Optional[torch.Tensor], logits: Optional[torch.Tensor], sg_col: int, top: int = 0) -> torch.Tensor:
+    """z[t] = sum_k w[t, k] D[pos[t, k]] + sigmoid(logits[t, sg_col]) * shared[t]  (sg_col < 0: ungated).
+    ``topk_w`` None (with ``top`` given): a plain sum, for experts whose weight scaled their input."""
+    top = topk_w.shape[1] if topk_w is not None else int(top)
+    if top <= 0 or pos_of_pair.numel() % top:
+        raise ValueError("moe_combine: the choices per token are needed")
+    if sg_col >= 0 and logits is None:
+        raise ValueError("moe_combine: a gated shared expert needs the router logits")
     if not _gpu(D, topk_w, shared):
-        return ref.moe_combine(D, pos_of_pair, topk_w, shared, logits, sg_col, D.dtype)
-    T, top = topk_w.shape
+        return ref.moe_combine(D, pos_of_pair, topk_w, shared, logits, sg_col, D.dtype, top)
+    T = pos_of_pair.numel() // top
     W = D.shape[1]
     z = torch.empty(T, W, dtype=D.dtype, device=D.device)
     _native().moe_combine(z.data_ptr(), _p(D), _p(pos_of_pair, I32), _p(topk_w, F32), _p(shared, D.dtype, "shared"),
-                          _p(logits, F32), logits.stride(0), sg_col, T, W, top, _f32(D.dtype), -1)
+                          _p(logits, F32), logits.stride(0) if logits is not None else 0, sg_col, T, W, top,
+                          _f32(D.dtype), -1)
     return z
+
+
+# ----------------------------------------------------------------------------- windowed attention with pooled blocks
+def pool_entries_per_page(block_size: int, P: int) -> int:
+    """Pooled blocks of P tokens that can start inside one cache page."""
+    return -(-block_size // P) if P > 0 else 0
+
+
+def window_kv_write(kcache: torch.Tensor, vcache: torch.Tensor, qkv: torch.Tensor, koff: int, voff: int,
+                    qb: Optional[torch.Tensor], kb: Optional[torch.Tensor], vb: Optional[torch.Tensor],
+                    cos_sin: Optional[torch.Tensor], positions: torch.Tensor, slot_mapping: torch.Tensor, H: int, G: int,
+                    D: int, V: int, dims: int, eps: float, unit: bool = True, *,
+                    vfirst_in: Optional[torch.Tensor] = None, vfirst_out: Optional[torch.Tensor] = None,
+                    lam: float = 0.0) -> None:
+    """Prepares a projected row [q (H D) | ... k (G D at ``koff``) ... v (G V at ``voff``) ...] of every token: biases,
+    rotation of the dimension pairs (2i, 2i + 1), i < dims / 2, by ``cos_sin[pos]`` = [cos | sin] (fp32), unit RMS per
+    head of q and k (``unit``), value mixing v <- (1 - lam) v + lam ``vfirst_in`` [T, G V] fp32; the first mixing layer
+    leaves its v in ``vfirst_out``.  q is rewritten in place; k and v go to the paged caches [slots, G, D] / [slots, G, V]."""
+    dt = qkv.dtype
+    if qkv.dim() != 2 or qkv.stride(1) != 1:
+        raise ValueError("window_kv_write: the projected rows must be contiguous")
+    if koff + G * D > qkv.shape[1] or voff + G * V > qkv.shape[1] or H * D > qkv.shape[1]:
+        raise ValueError("window_kv_write: part offsets exceed the projected row")
+    if not _gpu(kcache, vcache, qkv):
+        return ref.window_kv_write(kcache, vcache, qkv, koff, voff, qb, kb, vb, cos_sin, positions, slot_mapping,
+                                   vfirst_in, vfirst_out, lam, H, G, D, V, dims, eps, unit)
+    T = qkv.shape[0]
+    if cos_sin is not None and (cos_sin.shape[1] != dims or cos_sin.dtype != F32):
+        raise ValueError("window_kv_write: the angle table must be fp32 [positions, dims]")
+    for t in (vfirst_in, vfirst_out):
+        if t is not None and (t.shape != (T, G * V) or t.dtype != F32):
+            raise ValueError("window_kv_write: mixed values are fp32 [T, G V]")
+    _native().window_kv_write(_p(kcache, dt, "kcache"), _p(vcache, dt, "vcache"), qkv.data_ptr(), qkv.stride(0), koff,
+                              voff, _p(qb, dt, "qb"), _p(kb, dt, "kb"), _p(vb, dt, "vb"), _p(cos_sin),
+                              _p(positions, I32), _p(slot_mapping, I32), _p(vfirst_in), _p(vfirst_out), float(lam), T, H,
+                              G, D, V, dims, float(eps), int(bool(unit)), _f32(dt), -1)
+
+
+def window_pool(kpool: torch.Tensor, vpool: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+                block_tables: torch.Tensor, tok_seq: torch.Tensor, positions: torch.Tensor, P: int,
+                block_size: int) -> None:
+    """For every token of the batch that ends a block of P tokens ((pos + 1) % P == 0): the fp32 mean of the block's
+    cached keys / values -> kpool / vpool [pages * ceil(block_size / P), G, D or V] (the block's entry lives with the
+    page of its first token).  Call after :func:`window_kv_write` of the same batch."""
+    if P <= 0:
+        return
+    if kpool.dtype != F32 or vpool.dtype != F32:
+        raise TypeError("pooled keys / values are fp32")
+    if not _gpu(kpool, vpool, kcache, vcache):
+        return ref.window_pool(kpool, vpool, kcache, vcache, block_tables, tok_seq, positions, P, block_size)
+    G, D, V = kcache.shape[1], kcache.shape[2], vcache.shape[2]
+    _native().window_pool(_p(kpool), _p(vpool), _p(kcache), _p(vcache, kcache.dtype, "vcache"),
+                          _p(block_tables, I32, "block_tables"), block_tables.shape[1], _p(tok_seq, I32),
+                          _p(positions, I32), positions.shape[0], G, D, V, P, block_size, _f32(kcache.dtype), -1)
+
+
+def window_attention(q: torch.Tensor, gate: Optional[torch.Tensor], kcache: torch.Tensor, vcache: torch.Tensor,
+                     kpool: Optional[torch.Tensor], vpool: Optional[torch.Tensor], block_tables: torch.Tensor,
+                     tok_seq: torch.Tensor, positions: torch.Tensor, H: int, window: int, P: int, scale: float,
+                     sink: bool, block_size: int) -> torch.Tensor:
+    """Grouped-query attention over the paged caches [slots, G, D] / [slots, G, V]: the token at position p sees the
+    tokens max(0, p - window + 1) .. p (``window`` <= 0: all) and, with ``P`` > 0, the pooled blocks that lie wholly
+    before the window (b P + P - 1 <= p - window), all in one softmax; ``sink``: one more unit in the denominator.
+    ``q`` [T, >= H D] (row stride free, the prepared queries first), ``gate`` [T, H V] (row stride free): the result is
+    multiplied by sigmoid(gate).  Returns [T, H V]."""
+    G, D, V = kcache.shape[1], kcache.shape[2], vcache.shape[2]
+    if H % G:
+        raise ValueError(f"window_attention: {H} query heads over {G} key heads")
+    if window <= 0:
+        P = 0
+    if not _gpu(q, kcache, vcache):
+        return ref.window_attention(q, gate, kcache, vcache, kpool, vpool, block_tables, tok_seq, positions, H, G, D, V,
+                                    window, P, scale, sink, block_size, q.dtype)
+    T = q.shape[0]
+    dt = q.dtype
+    if q.stride(1) != 1 or (gate is not None and (gate.stride(1) != 1 or gate.dtype != dt)):
+        raise ValueError("window_attention: q and gate rows must be contiguous and of one dtype")
+    out = torch.empty(T, H * V, dtype=dt, device=q.device)
+    _native().window_attention(out.data_ptr(), q.data_ptr(), q.stride(0), gate.data_ptr() if gate is not None else 0,
+                               gate.stride(0) if gate is not None else 0, _p(kcache, dt, "kcache"),
+                               _p(vcache, dt, "vcache"), _p(kpool, F32, "kpool"), _p(vpool, F32, "vpool"),
+                               _p(block_tables, I32, "block_tables"), block_tables.shape[1], _p(tok_seq, I32),
+                               _p(positions, I32), T, H, G, D, V, int(window), int(P), float(scale), int(bool(sink)),
+                               block_size, _f32(dt), -1)
+    return out
+
+
+# ----------------------------------------------------------------------------- gated matrix-state recurrences
+def gated_scan_max_dim() -> int:
+    return 128
+
+
+def gated_scan_record(kind: int, D: int, V: int) -> int:
+    """fp32 values of one (slot, head) state record: S [D, V] (SCAN_MLSTM: then n [D] and the running maximum)."""
+    return ref.gated_scan_record(kind, D, V)
+
+
+def gated_scan(proj: torch.Tensor, kind: int, cols: dict, normw: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor,
+               seq_slots: torch.Tensor, positions: torch.Tensor, H: int, D: int, V: int, eps: float, out_dtype, *,
+               fbias: Optional[torch.Tensor] = None, ibias: Optional[torch.Tensor] = None,
+               lower: Optional[torch.Tensor] = None, cap: float = 0.0) -> torch.Tensor:
+    """A gated linear recurrence with a matrix state per head over a varlen batch; ``proj`` fp32 [T, ld] is the fused
+    input projection with its parts at the column offsets ``cols``; ``state`` [slots, H, record] fp32 is updated in
+    place (a portion at position 0 starts from zero).  Returns the normed (and, SCAN_MLSTM, gated) outputs [T, H V].
+    SCAN_HGRN2: cols q, f, v; ``lower`` [H D], ``fbias`` [H D], ``normw`` [V].
+    SCAN_MLSTM: cols q, k, v, i, f, g; ``ibias`` / ``fbias`` [H], ``cap`` > 0, ``normw`` [H V]."""
+    if proj.dtype != F32 or state.dtype != F32:
+        raise TypeError("the recurrence's inputs and state are fp32")
+    if proj.dim() != 2 or proj.stride(1) != 1:
+        raise ValueError("gated_scan: projected rows must be contiguous")
+    need = {SCAN_HGRN2: ("q", "f", "v"), SCAN_MLSTM: ("q", "k", "v", "i", "f", "g")}[kind]
+    width = {"q": H * D, "k": H * D, "v": H * V, "g": H * V, "i": H, "f": H * D if kind == SCAN_HGRN2 else H}
+    for key in need:
+        if cols[key] < 0 or cols[key] + width[key] > proj.shape[1]:
+            raise ValueError(f"gated_scan: part {key!r} exceeds the projected row")
+    if state.shape[1:] != (H, gated_scan_record(kind, D, V)):
+        raise ValueError("gated_scan: state must be [slots, H, record]")
+    if not _gpu(proj, state):
+        return ref.gated_scan(proj, kind, cols, fbias, ibias, lower, normw, state, cu_q, seq_slots, positions, H, D, V,
+                              eps, cap, out_dtype)
+    if max(D, V) > gated_scan_max_dim():
+        raise ValueError(f"gated_scan: head sizes {D} x {V} exceed the kernel's {gated_scan_max_dim()}")
+    T = proj.shape[0]
+    out = torch.empty(T, H * V, dtype=out_dtype, device=proj.device)
+    c = lambda key: int(cols.get(key, 0))
+    _native().gated_scan(out.data_ptr(), _p(proj), proj.stride(0), kind, c("q"), c("k"), c("v"), c("i"), c("f"), c("g"),
+                         _p(fbias, out_dtype, "fbias"), _p(ibias, out_dtype, "ibias"), _p(lower, out_dtype, "lower"),
+                         _p(normw, out_dtype, "normw"), _p(state), _p(cu_q, I32), _p(seq_slots, I32),
+                         _p(positions, I32), cu_q.shape[0] - 1, H, D, V, float(eps), float(cap), _f32(out_dtype), -1)
+    return out
