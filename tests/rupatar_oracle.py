@@ -196,3 +196,13 @@ def forward(tokens: List[int], tensors: Dict[str, torch.Tensor], config: dict, r
         after.append(x.clone())
     hf = group_norm(x, _w(tensors, "final.norm"), groups, eps)
     return hf @ _w(tensors, "head").T, after
+
+
+def greedy(prompt: List[int], tensors, config: dict, n: int) -> List[int]:
+    """n tokens of greedy continuation (the whole sequence is recomputed for every token)."""
+    toks, out = list(prompt), []
+    for _ in range(n):
+        logits, _ = forward(toks, tensors, config)
+        out.append(int(torch.argmax(logits[-1])))
+        toks.append(out[-1])
+    return out
