@@ -76,7 +76,9 @@ def main() -> int:
                          "decode graphs with the top-p passes")
     ap.add_argument("--model-bench", action="store_true",
                     help="instead of the headline workload: prefill / decode tokens/s of the registered model designs "
-                         "(Putulorn dense, Putulorn with experts, Llama) at equal layer sizes, random weights")
+                         "(Putulorn dense, Putulorn with experts, Rupatar, Llama) at equal layer sizes, random weights")
+    ap.add_argument("--model-bench-models", default="",
+                    help="(--model-bench) only these rows, comma-separated: putulorn-dense, putulorn-moe, rupatar, llama")
     ap.add_argument("--model-bench-widths", default="2048,4096", help="(--model-bench) model widths, comma-separated")
     ap.add_argument("--verbose", action="store_true", help="engine INFO logs (init, autotune, graph capture)")
     args = ap.parse_args()
@@ -84,7 +86,9 @@ def main() -> int:
     if args.model_bench:
         from k8s_llm_scheduler_amd.engine import modelbench
 
-        rows = modelbench.run(widths=tuple(int(w) for w in args.model_bench_widths.split(",")), progress=lambda r: print(json.dumps(r), file=sys.stderr, flush=True))
+        rows = modelbench.run(widths=tuple(int(w) for w in args.model_bench_widths.split(",")),
+                              models=tuple(m for m in args.model_bench_models.split(",") if m) or None,
+                              progress=lambda r: print(json.dumps(r), file=sys.stderr, flush=True))
         print(json.dumps({"metric": "model_bench", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic",
                           "rows": rows}))
         return 0

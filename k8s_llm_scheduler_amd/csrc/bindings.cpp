@@ -153,6 +153,11 @@ int k8s_window_attention(void* out, const void* q, long ldq, const void* gate, l
                          const void* vcache, const float* kpool, const float* vpool, const int* block_tables,
                          int max_blocks, const int* tok_seq, const int* positions, int T, int H, int G, int D, int V,
                          int window, int P, float scale, int sink, int bs, int f32, hipStream_t s);
+int k8s_window_mfma_ok(int H, int G, int D, int V);
+int k8s_window_attention_mfma(void* out, const void* q, long ldq, const void* gate, long ldg, const void* kcache,
+                              const void* vcache, const float* kpool, const float* vpool, const int* block_tables,
+                              int max_blocks, const int* cu_q, const int* positions, int nseq, int max_qlen, int H, int G,
+                              int D, int V, int window, int P, float scale, int sink, int bs, hipStream_t s);
 int k8s_gated_scan_max_dim();
 long long k8s_gated_scan_record(int kind, int D, int V);
 int k8s_gated_scan(void* out, const float* proj, long ld, int kind, int cq, int ck, int cv, int ci, int cf, int cg,
@@ -491,6 +496,15 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
     check(k8s_window_attention(P(out), P(q), ldq, P(gate), ldg, P(kcache), P(vcache), P<float>(kpool), P<float>(vpool),
                                P<int>(bt), max_blocks, P<int>(tok_seq), P<int>(positions), T, H, G, D, V, window, P_,
                                scale, sink, bs, f32, S(s)), "window_attention");
+  });
+  m.def("window_mfma_ok", [](int H, int G, int D, int V) { return k8s_window_mfma_ok(H, G, D, V) != 0; });
+  m.def("window_attention_mfma", [](uintptr_t out, uintptr_t q, long ldq, uintptr_t gate, long ldg, uintptr_t kcache,
+                                    uintptr_t vcache, uintptr_t kpool, uintptr_t vpool, uintptr_t bt, int max_blocks,
+                                    uintptr_t cu_q, uintptr_t positions, int nseq, int max_qlen, int H, int G, int D,
+                                    int V, int window, int P_, float scale, int sink, int bs, int64_t s) {
+    check(k8s_window_attention_mfma(P(out), P(q), ldq, P(gate), ldg, P(kcache), P(vcache), P<float>(kpool),
+                                    P<float>(vpool), P<int>(bt), max_blocks, P<int>(cu_q), P<int>(positions), nseq,
+                                    max_qlen, H, G, D, V, window, P_, scale, sink, bs, S(s)), "window_attention_mfma");
   });
   m.def("gated_scan_max_dim", []() { return k8s_gated_scan_max_dim(); });
   m.def("gated_scan_record", [](int kind, int D, int V) { return k8s_gated_scan_record(kind, D, V); });

@@ -219,6 +219,226 @@ __global__ void window_attention_kernel(TA* __restrict__ out, const TA* __restri
   }
 }
 
+
+// The same attention on the matrix cores for prompts in bf16 (D % 8 == 0, V % 16 == 0, R = H / G a power of two <= 16).
+// A workgroup of 4 waves takes TPB consecutive tokens of one sequence and one key / value head; a wave owns NCB blocks
+// of 16 query columns, a column being one (token, query head of the group) pair, 16 / R tokens per block.  The keys of
+// the workgroup are the ordered list [pooled blocks 0 .. nb(last token) | tokens lo(first token) .. last token]; 32 of
+// them per step are staged in LDS as bf16 (pooled rows converted from fp32) and shared by the waves, each column masks
+// what its own token does not see:
+//   S^T[key][column] = K Q^T      A = 16 staged key rows, B = the columns' queries (registers)
+//   O[column][d]    += P V        A = the 32 keys' probabilities (registers, keys in the order the S^T tiles left
+//                                 them), B = the staged value columns through the transposing LDS read
+// scores, softmax and sums in fp32; a sink starts every column at (max 0, sum 1).
+typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
+
+template <int NKK, int NVB, int NCB>
+__global__ __launch_bounds__(256) void window_attention_mfma_kernel(
+    bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long ldq, const bf16_t* __restrict__ gate, long ldg,
+    const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache, const float* __restrict__ kpool,
+    const float* __restrict__ vpool, const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
+    const int* __restrict__ positions, int H, int G, int D, int V, int window, int P, float scale, int sink, int bs,
+    int ppb, int R) {
+  extern __shared__ __attribute__((aligned(16))) char smem_w[];
+  const int seq = blockIdx.z, g = blockIdx.y;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 15, g4 = lane >> 4;
+  const int TPC = 16 / R, TPB = 4 * NCB * TPC;
+  const int tq0 = cu_q[seq] + blockIdx.x * TPB, tend = cu_q[seq + 1];
+  if (tq0 >= tend) return;
+  const int p_first = positions[tq0];
+  const int nval = min(TPB, tend - tq0);
+  if (p_first < 0) {   // idle rows: defined output
+    for (int i = tid; i < nval * R * V; i += 256) {
+      const int tt = i / (R * V), r = i - tt * (R * V);
+      out[(size_t)(tq0 + tt) * H * V + (size_t)g * R * V + r] = 0;
+    }
+    return;
+  }
+  const int p_last = p_first + nval - 1;
+  const int rowk = (D + 8) * 2, rowv = (V + 8) * 2;      // LDS row bytes
+  char* klds = smem_w;                                   // [32][D + 8] bf16
+  char* vlds = smem_w + 32 * rowk;                       // [32][V + 8] bf16
+  const bool win = window > 0;
+  const int lo_min = win ? max(0, p_first - window + 1) : 0;
+  const int nb_max = (win && P > 0 && p_last - window + 1 >= P) ? (p_last - window + 1) / P : 0;
+  const int nkeys = nb_max + (p_last + 1 - lo_min);
+  const int nsteps = (nkeys + 31) / 32;
+  const int* btr = block_tables + (size_t)seq * max_blocks;
+  const int GD = G * D, GV = G * V;
+  const int ckd = D / 8, ckv = V / 8, cpr = ckd + ckv;   // 16-byte chunks per staged row
+  const int nkk = (D + 31) / 32, nvb = V / 16;
+  const u32x4 zero = u32x4{0u, 0u, 0u, 0u};
+  // this lane's column in every block of the wave: token, position, first visible token, visible pooled blocks
+  int c_tok[NCB], c_p[NCB], c_lo[NCB], c_nb[NCB];
+  bf16x8 qf[NCB][NKK];
+  int w_pmin = 0x7fffffff, w_pmax = -1;
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) {
+    const int toff = (wave * NCB + cb) * TPC + li / R;
+    const bool ok = toff < nval;
+    c_tok[cb] = tq0 + toff;
+    c_p[cb] = ok ? p_first + toff : -1;
+    c_lo[cb] = win ? max(0, c_p[cb] - window + 1) : 0;
+    c_nb[cb] = (ok && win && P > 0 && c_p[cb] - window + 1 >= P) ? (c_p[cb] - window + 1) / P : 0;
+    const int hd = g * R + li % R;
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {
+      const int piece = 32 * kk + 8 * g4;
+      u32x4 v = zero;
+      if (ok && piece < D) v = *reinterpret_cast<const u32x4*>(q + (size_t)c_tok[cb] * ldq + (size_t)hd * D + piece);
+      qf[cb][kk] = __builtin_bit_cast(bf16x8, v);
+    }
+    const int t_lo = (wave * NCB + cb) * TPC, t_hi = min(t_lo + TPC, nval) - 1;
+    if (t_lo < nval) {
+      w_pmin = min(w_pmin, p_first + t_lo);
+      w_pmax = max(w_pmax, p_first + t_hi);
+    }
+  }
+  const bool w_any = w_pmax >= 0;
+  const int w_lo = (w_any && win) ? max(0, w_pmin - window + 1) : 0;
+  const int w_nb = (w_any && win && P > 0 && w_pmax - window + 1 >= P) ? (w_pmax - window + 1) / P : 0;
+  f32x4 o[NCB][NVB];
+  float m_run[NCB], l_run[NCB];
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) {
+    m_run[cb] = sink ? 0.f : -INFINITY;
+    l_run[cb] = sink ? 1.f : 0.f;
+#pragma unroll
+    for (int n = 0; n < NVB; ++n) o[cb][n] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const int qd = li >> 2, pd = li & 3;
+  for (int step = 0; step < nsteps; ++step) {
+    const int u0 = step * 32;
+    __syncthreads();
+    for (int idx = tid; idx < 32 * cpr; idx += 256) {
+      const int r = idx / cpr, c = idx - r * cpr, u = u0 + r;
+      const bool isk = c < ckd;
+      const int e8 = 8 * (isk ? c : c - ckd);
+      u32x4 v = zero;
+      if (u < nb_max) {
+        const size_t e = pool_entry(btr, u, P, bs, ppb);
+        const float* src = isk ? kpool + e * GD + (size_t)g * D + e8 : vpool + e * GV + (size_t)g * V + e8;
+        const f32x4 a = *reinterpret_cast<const f32x4*>(src), b = *reinterpret_cast<const f32x4*>(src + 4);
+        v = u32x4{pack_bf2(a[0], a[1]), pack_bf2(a[2], a[3]), pack_bf2(b[0], b[1]), pack_bf2(b[2], b[3])};
+      } else if (u < nkeys) {
+        const int j = lo_min + (u - nb_max);
+        const size_t slot = (size_t)btr[j / bs] * bs + (j % bs);
+        v = isk ? *reinterpret_cast<const u32x4*>(kcache + slot * GD + (size_t)g * D + e8)
+                : *reinterpret_cast<const u32x4*>(vcache + slot * GV + (size_t)g * V + e8);
+      }
+      *reinterpret_cast<u32x4*>((isk ? klds + r * rowk : vlds + r * rowv) + 2 * e8) = v;
+    }
+    __syncthreads();
+    // keys of this step that any column of the wave can see: pooled blocks below w_nb, tokens w_lo .. w_pmax
+    bool any = false;
+    if (w_any) {
+      if (u0 < nb_max) any = u0 < w_nb;
+      const int j_first = lo_min + max(u0 - nb_max, 0), j_last = lo_min + (u0 + 31 - nb_max);
+      if (u0 + 31 >= nb_max && j_first <= w_pmax && j_last >= w_lo) any = true;
+    }
+    if (!any) continue;
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) {
+      f32x4 sacc[2];
+#pragma unroll
+      for (int m = 0; m < 2; ++m) {
+        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < NKK; ++kk) {
+          if (kk < nkk) {
+            const int piece = 32 * kk + 8 * g4;
+            bf16x8 ka = __builtin_bit_cast(bf16x8, zero);
+            if (piece < D) ka = *reinterpret_cast<const bf16x8*>(klds + (16 * m + li) * rowk + 2 * piece);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[cb][kk], acc, 0, 0, 0);
+          }
+        }
+        sacc[m] = acc;   // S[key u0 + 16 m + 4 g4 + i][column li]
+      }
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int u = u0 + 16 * m + 4 * g4 + i;
+          bool vis;
+          if (u < nb_max) vis = u < c_nb[cb];
+          else {
+            const int j = lo_min + (u - nb_max);
+            vis = j <= c_p[cb] && j >= c_lo[cb];
+          }
+          const float v = vis ? sacc[m][i] * scale : -INFINITY;
+          sacc[m][i] = v;
+          tmax = fmaxf(tmax, v);
+        }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+      const float m_new = fmaxf(m_run[cb], tmax);
+      const float m_ref = m_new == -INFINITY ? 0.f : m_new;      // a column that has seen nothing yet
+      const float alpha = m_run[cb] == -INFINITY ? 0.f : expf(m_run[cb] - m_ref);
+      float rsum = 0.f;
+#pragma unroll
+      for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float pv = expf(sacc[m][i] - m_ref);
+          sacc[m][i] = pv;
+          rsum += pv;
+        }
+      rsum += __shfl_xor(rsum, 16, WAVE);
+      rsum += __shfl_xor(rsum, 32, WAVE);
+      l_run[cb] = l_run[cb] * alpha + rsum;
+      m_run[cb] = m_new;
+      float a_i[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a_i[i] = __shfl(alpha, g4 * 4 + i, WAVE);
+      bf16x8 pa;       // slot j < 4: key 4 g4 + j; slot j >= 4: key 16 + 4 g4 + (j - 4)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        pa[j] = (__bf16)sacc[0][j];
+        pa[4 + j] = (__bf16)sacc[1][j];
+      }
+      const int r0 = 4 * g4 + qd, r1 = r0 + 16;
+#pragma unroll
+      for (int n = 0; n < NVB; ++n) {
+        if (n < nvb) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[cb][n][i] *= a_i[i];
+          const int col = 16 * n + 4 * pd;
+          const bf16x4 v0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(vlds + r0 * rowv + 2 * col));
+          const bf16x4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(vlds + r1 * rowv + 2 * col));
+          bf16x8 vb;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) { vb[j] = v0[j]; vb[4 + j] = v1[j]; }
+          o[cb][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vb, o[cb][n], 0, 0, 0);
+        }
+      }
+    }
+  }
+  // o[cb][n][i] = O[column 4 g4 + i][d 16 n + li]; a column's sum lives in the lanes with li == column
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) {
+    float l_i[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) l_i[i] = __shfl(l_run[cb], g4 * 4 + i, WAVE);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = 4 * g4 + i;
+      const int toff = (wave * NCB + cb) * TPC + c / R;
+      if (toff >= nval) continue;
+      const int t = tq0 + toff, hd = g * R + c % R;
+      const float inv = 1.f / l_i[i];
+#pragma unroll
+      for (int n = 0; n < NVB; ++n)
+        if (n < nvb) {
+          const int d = 16 * n + li;
+          float y = o[cb][n][i] * inv;
+          if (gate != nullptr) y *= 1.f / (1.f + expf(-bf2f(gate[(size_t)t * ldg + (size_t)hd * V + d])));
+          out[(size_t)t * H * V + (size_t)hd * V + d] = f2bf(y);
+        }
+    }
+  }
+}
+
 }  // namespace k8sllm
 
 using namespace k8sllm;
@@ -287,5 +507,37 @@ extern "C" int k8s_window_attention(void* out, const void* q, long ldq, const vo
   else K8S_WA_T(bf16_t);
 #undef K8S_WA_T
 #undef K8S_WA
+  return (int)hipGetLastError();
+}
+
+// Whether the matrix-core kernel takes these sizes (else the caller uses k8s_window_attention).
+extern "C" int k8s_window_mfma_ok(int H, int G, int D, int V) {
+  if (G <= 0 || H % G) return 0;
+  const int R = H / G;
+  return (R == 1 || R == 2 || R == 4 || R == 8 || R == 16) && D % 8 == 0 && V % 16 == 0 && D <= 256 && V <= 256;
+}
+
+// Prompt portions in bf16: nseq sequences of at most max_qlen tokens, cu_q their query offsets.
+extern "C" int k8s_window_attention_mfma(void* out, const void* q, long ldq, const void* gate, long ldg,
+                                         const void* kcache, const void* vcache, const float* kpool, const float* vpool,
+                                         const int* block_tables, int max_blocks, const int* cu_q, const int* positions,
+                                         int nseq, int max_qlen, int H, int G, int D, int V, int window, int P,
+                                         float scale, int sink, int bs, hipStream_t s) {
+  if (nseq <= 0 || max_qlen <= 0) return 0;
+  if (!k8s_window_mfma_ok(H, G, D, V) || bs <= 0 || nseq > 65535 || G > 65535 || ldq % 8 || ((uintptr_t)q & 15)) return -1;
+  if (window > 0 && P > 0 && (kpool == nullptr || vpool == nullptr)) return -1;
+  const int R = H / G, ppb = P > 0 ? (bs + P - 1) / P : 1;
+  const size_t lds = (size_t)32 * ((D + 8) + (V + 8)) * 2;
+  constexpr int NCB = 2;
+  const int TPB = 4 * NCB * (16 / R);
+  const dim3 grid((max_qlen + TPB - 1) / TPB, G, nseq);
+#define K8S_WM(NKK, NVB)                                                                                              \
+  window_attention_mfma_kernel<NKK, NVB, NCB><<<grid, 256, lds, s>>>(                                                 \
+      (bf16_t*)out, (const bf16_t*)q, ldq, (const bf16_t*)gate, ldg, (const bf16_t*)kcache, (const bf16_t*)vcache,    \
+      kpool, vpool, block_tables, max_blocks, cu_q, positions, H, G, D, V, window, P, scale, sink, bs, ppb, R)
+  if (D <= 64 && V <= 64) K8S_WM(2, 4);
+  else if (D <= 128 && V <= 128) K8S_WM(4, 8);
+  else K8S_WM(8, 16);
+#undef K8S_WM
   return (int)hipGetLastError();
 }

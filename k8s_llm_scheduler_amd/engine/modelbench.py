@@ -1,7 +1,8 @@
 """Prefill and decode throughput of the registered model designs at equal layer sizes (``bench.py --model-bench``).
 
-For every size a Putulorn (dense feed-forwards), a Putulorn with experts and a Llama of the same width, depth,
-feed-forward size and vocabulary are built with random weights and driven through the same engine entry points:
+For every size a Putulorn (dense feed-forwards), a Putulorn with experts, a Rupatar (experts in every layer) and a Llama
+of the same width, depth, feed-forward / expert size and vocabulary are built with random weights and driven through the
+same engine entry points:
 
 * prefill: one whole prompt of ``T`` tokens in one step (``LLMEngine.replay_step``, the varlen forward), tokens/s;
 * decode: ``B`` requests generated together (``LLMEngine.generate``: captured decode graphs), new tokens/s from the
@@ -22,12 +23,19 @@ VOCAB = 32768
 
 
 def _register(width: int) -> Dict[str, str]:
-    from ..models import putulorn
+    from ..models import putulorn, rupatar
     from ..models.config import PRESETS, LlamaConfig
 
     pairs, ff, wd, heads, eff, experts = SIZES[width]
     names = {"putulorn-dense": f"putulorn-w{width}-dense", "putulorn-moe": f"putulorn-w{width}-moe",
-             "llama": f"llama-w{width}"}
+             "rupatar": f"rupatar-w{width}", "llama": f"llama-w{width}"}
+    # Rupatar: 2 x pairs layers in the order attention, hgrn2, attention, mlstm (windowed attention with 4 query heads
+    # per key head, window 1024, pooled blocks of 16; recurrences of head size 64 x 64 like the wkv heads), every layer
+    # with the experts of the Putulorn-moe layers and a shared expert of the same size
+    rupatar.PRESETS[names["rupatar"]] = rupatar.preset(
+        names["rupatar"], width, VOCAB, max(1, pairs // 2), heads=heads, kv_heads=heads // 4, dim=128, vdim=128,
+        window=1024, pool=16, rot_dims=64, scan_heads=width // wd, scan_dim=wd, scan_vdim=wd, experts=experts, top=2,
+        expert_ff=eff, shared_ff=eff)
     kw = dict(heads=heads, wkv_dim=wd, dim=128, rot_dim=64, vdim=128, kv_rank=512, window=1024, ff=ff)
     putulorn.PRESETS[names["putulorn-dense"]] = putulorn.preset(names["putulorn-dense"], width, VOCAB, pairs, **kw)
     putulorn.PRESETS[names["putulorn-moe"]] = putulorn.preset(names["putulorn-moe"], width, VOCAB, pairs, experts=experts,
@@ -38,7 +46,7 @@ def _register(width: int) -> Dict[str, str]:
 
 
 def run(widths=(2048, 4096), prefill_tokens=(512, 2048), decode_batches=(1, 8, 32), context: int = 512,
-        new_tokens: int = 32, repeats: int = 3, progress=print) -> List[dict]:
+        new_tokens: int = 32, repeats: int = 3, progress=print, models=None) -> List[dict]:
     import torch
 
     from . import build_engine
@@ -47,6 +55,8 @@ def run(widths=(2048, 4096), prefill_tokens=(512, 2048), decode_batches=(1, 8, 3
     rows = []
     for width in widths:
         for kind, name in _register(width).items():
+            if models and kind not in models:
+                continue
             maxb = max(decode_batches)
             mml = max(max(prefill_tokens), context + new_tokens + 16)
             eng = build_engine(name, max_batch=maxb, block_size=16, num_blocks=maxb * (mml // 16 + 1),

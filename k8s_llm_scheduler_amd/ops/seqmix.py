@@ -426,15 +426,21 @@ def window_pool(kpool: torch.Tensor, vpool: torch.Tensor, kcache: torch.Tensor, 
                           _p(positions, I32), positions.shape[0], G, D, V, P, block_size, _f32(kcache.dtype), -1)
 
 
+WINDOW_MFMA = os.environ.get("K8S_WINDOW_MFMA", "1") != "0"   # 0: always the plain-FMA attention kernel
+
+
 def window_attention(q: torch.Tensor, gate: Optional[torch.Tensor], kcache: torch.Tensor, vcache: torch.Tensor,
                      kpool: Optional[torch.Tensor], vpool: Optional[torch.Tensor], block_tables: torch.Tensor,
                      tok_seq: torch.Tensor, positions: torch.Tensor, H: int, window: int, P: int, scale: float,
-                     sink: bool, block_size: int) -> torch.Tensor:
+                     sink: bool, block_size: int, cu_q: Optional[torch.Tensor] = None, max_qlen: int = 0) -> torch.Tensor:
     """Grouped-query attention over the paged caches [slots, G, D] / [slots, G, V]: the token at position p sees the
     tokens max(0, p - window + 1) .. p (``window`` <= 0: all) and, with ``P`` > 0, the pooled blocks that lie wholly
     before the window (b P + P - 1 <= p - window), all in one softmax; ``sink``: one more unit in the denominator.
     ``q`` [T, >= H D] (row stride free, the prepared queries first), ``gate`` [T, H V] (row stride free): the result is
-    multiplied by sigmoid(gate).  Returns [T, H V]."""
+    multiplied by sigmoid(gate).  Returns [T, H V].
+    ``cu_q`` / ``max_qlen`` (the sequences' query offsets and longest portion): bf16 portions of prompts whose sizes
+    fit run on the matrix cores, tiles of consecutive tokens sharing the staged keys; anything else (fp32, single
+    tokens, other sizes) on the plain-FMA kernel."""
     G, D, V = kcache.shape[1], kcache.shape[2], vcache.shape[2]
     if H % G:
         raise ValueError(f"window_attention: {H} query heads over {G} key heads")
@@ -448,6 +454,16 @@ def window_attention(q: torch.Tensor, gate: Optional[torch.Tensor], kcache: torc
     if q.stride(1) != 1 or (gate is not None and (gate.stride(1) != 1 or gate.dtype != dt)):
         raise ValueError("window_attention: q and gate rows must be contiguous and of one dtype")
     out = torch.empty(T, H * V, dtype=dt, device=q.device)
+    nat = _native()
+    if (WINDOW_MFMA and dt == BF16 and cu_q is not None and max_qlen > 1 and nat.window_mfma_ok(H, G, D, V)
+            and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0):
+        nat.window_attention_mfma(out.data_ptr(), q.data_ptr(), q.stride(0), gate.data_ptr() if gate is not None else 0,
+                                  gate.stride(0) if gate is not None else 0, _p(kcache, dt, "kcache"),
+                                  _p(vcache, dt, "vcache"), _p(kpool, F32, "kpool"), _p(vpool, F32, "vpool"),
+                                  _p(block_tables, I32, "block_tables"), block_tables.shape[1], _p(cu_q, I32, "cu_q"),
+                                  _p(positions, I32), cu_q.shape[0] - 1, int(max_qlen), H, G, D, V, int(window), int(P),
+                                  float(scale), int(bool(sink)), block_size, -1)
+        return out
     _native().window_attention(out.data_ptr(), q.data_ptr(), q.stride(0), gate.data_ptr() if gate is not None else 0,
                                gate.stride(0) if gate is not None else 0, _p(kcache, dt, "kcache"),
                                _p(vcache, dt, "vcache"), _p(kpool, F32, "kpool"), _p(vpool, F32, "vpool"),

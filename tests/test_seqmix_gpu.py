@@ -213,3 +213,161 @@ def test_grouped_gemm_many_rows():
     want = sm.gemm(h, w, a_rows=stc, tiles=tilesc, rows=Tn * top, seg=segc).float()
     # rows of an expert may come in another order: compare per (token, choice) pair
     close(got[pos.cpu().long()], want[posc.long()], 2e-2)
+
+
+# ----------------------------------------------------------------------------- grouped norm, row-scaled gelu, sigmoid router
+@pytest.mark.parametrize("dt,tol", DTYPES)
+def test_grouped_norm_scaled_embedding_and_row_factors(dt, tol):
+    torch.manual_seed(20)
+    W = 240
+    ids = torch.randint(0, 50, (T,), dtype=torch.int32)
+    table = torch.randn(50, W).to(dt)
+    close(sm.embed_rows(ids.to(DEV), table.to(DEV), 3.7), sm.embed_rows(ids, table, 3.7), 1e-6)
+    for groups in (2, 5, 8, 240):
+        x, br, rv, w = torch.randn(T, W), torch.randn(T, W).to(dt), torch.randn(W).to(dt), torch.randn(W).to(dt)
+        xg, xc = x.to(DEV).clone(), x.clone()
+        og = sm.resnorm(xg, w.to(DEV), 1e-6, branch=br.to(DEV), rowvec=rv.to(DEV), out_dtype=dt, groups=groups)
+        oc = sm.resnorm(xc, w, 1e-6, branch=br, rowvec=rv, out_dtype=dt, groups=groups)
+        close(og, oc, tol)
+        close(xg, xc, 1e-6)
+    a = (torch.randn(T, 70) * 2).to(dt)
+    close(sm.act(a.to(DEV), sm.ACT_GELU_ERF), sm.act(a, sm.ACT_GELU_ERF), tol)
+    sc, perm = torch.rand(T) * 2, torch.randperm(T).int()
+    close(sm.act(a.to(DEV), sm.ACT_GELU_ERF, row_scale=sc.to(DEV), row_map=perm.to(DEV)),
+          sm.act(a, sm.ACT_GELU_ERF, row_scale=sc, row_map=perm), tol)
+    close(sm.act(a.to(DEV), sm.ACT_SILU, row_scale=sc.to(DEV)), sm.act(a, sm.ACT_SILU, row_scale=sc), tol)
+
+
+@pytest.mark.parametrize("E,top", [(8, 2), (70, 4), (5, 5), (3, 1)])
+def test_sigmoid_router_and_plain_combine(E, top):
+    torch.manual_seed(21)
+    logits = torch.randn(T, E + 1) * 2
+    ig, wg = sm.moe_route(logits.to(DEV), E, top, 1.0, score="sigmoid")
+    ic, wc = sm.moe_route(logits, E, top, 1.0, score="sigmoid")
+    assert torch.equal(ig.cpu(), ic)
+    close(wg, wc, 1e-6)
+    assert torch.allclose(wc, torch.sigmoid(logits[:, :E]).gather(1, ic.long()))
+    D = torch.randn(T * top, 24)
+    pos = torch.randperm(T * top).int()
+    shared = torch.randn(T, 24)
+    close(sm.moe_combine(D.to(DEV), pos.to(DEV), None, shared.to(DEV), None, -1, top=top),
+          sm.moe_combine(D, pos, None, shared, None, -1, top=top), 1e-6)
+    close(sm.moe_combine(D.to(DEV), pos.to(DEV), None, None, None, -1, top=top),
+          sm.moe_combine(D, pos, None, None, None, -1, top=top), 1e-6)
+
+
+# ----------------------------------------------------------------------------- windowed attention with pooled blocks
+def window_case(H, G, D, V, window, P, dims, dt, bs=16, seed=0):
+    """Three sequences over shuffled pages: a prompt from 0, a portion that resumes at position 70 and a single token at
+    position 130; their earlier tokens are written to the caches first (in two batches, so pooled blocks straddle
+    them)."""
+    torch.manual_seed(seed)
+    nblk = 40
+    lens = [(0, 90), (70, 55), (130, 1)]
+    perm = torch.randperm(nblk).int()
+    bt = torch.zeros(3, 12, dtype=torch.int32)
+    for s in range(3):
+        bt[s] = perm[12 * s:12 * s + 12]
+    ncol = H * D + G * D + G * V + H * V
+    cs = ref.rope_table(dims, 256, 1000.0, {"type": "linear", "factor": 2.0}) if dims else None
+
+    def rows(n):
+        return (torch.randn(n, ncol) * 0.7).to(dt)
+
+    def meta(spans):
+        cu, pos, tok_seq, slots = [0], [], [], []
+        for s, (a, n) in spans:
+            cu.append(cu[-1] + n)
+            pos += range(a, a + n)
+            tok_seq += [s] * n
+            slots += [int(bt[s, p // bs]) * bs + p % bs for p in range(a, a + n)]
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32)
+        return i32(cu), i32(pos), i32(tok_seq), i32(slots)
+
+    qb, kb, vb = (torch.randn(n).to(dt) * 0.3 for n in (H * D, G * D, G * V))
+    e = nblk * sm.pool_entries_per_page(bs, P) if P else 1
+    caches = {}
+    for dev in ("cpu", DEV):
+        kc, vc = torch.zeros(nblk * bs, G, D, dtype=dt, device=dev), torch.zeros(nblk * bs, G, V, dtype=dt, device=dev)
+        kp, vp = torch.zeros(e, G, D, device=dev), torch.zeros(e, G, V, device=dev)
+        caches[dev] = (kc, vc, kp, vp)
+    batches = [meta([(1, (0, 41)), (2, (0, 77))]), meta([(1, (41, 29)), (2, (77, 53))]),
+               meta([(s, l) for s, l in enumerate(lens)])]
+    outs = {}
+    for dev in ("cpu", DEV):
+        kc, vc, kp, vp = caches[dev]
+        mv = lambda t: None if t is None else t.to(dev)
+        torch.manual_seed(seed + 1)
+        for cu, pos, tok_seq, slots in batches:
+            x = rows(pos.shape[0]).to(dev)
+            vfirst = (torch.randn(pos.shape[0], G * V)).to(dev)
+            sm.window_kv_write(kc, vc, x, H * D, H * D + G * D, mv(qb), mv(kb), mv(vb), mv(cs), pos.to(dev), slots.to(dev),
+                               H, G, D, V, dims, 1e-6, True, vfirst_in=vfirst, lam=0.3)
+            sm.window_pool(kp, vp, kc, vc, bt.to(dev), tok_seq.to(dev), pos.to(dev), P, bs)
+        goff = H * D + G * D + G * V
+        outs[dev] = (x, sm.window_attention(x, x[:, goff:], kc, vc, kp if P else None, vp if P else None, bt.to(dev),
+                                            tok_seq.to(dev), pos.to(dev), H, window, P, 0.35, True, bs, cu.to(dev),
+                                            max(n for _, n in lens)))
+    return outs, caches
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+@pytest.mark.parametrize("H,G,D,V,window,P,dims", [
+    (4, 2, 24, 20, 33, 5, 8),        # odd sizes: the plain kernel in both types
+    (6, 2, 16, 16, 20, 16, 16),      # three query heads per key head: no matrix-core tiling
+    (8, 2, 64, 64, 40, 12, 32),      # matrix cores in bf16: four query heads per key head
+    (4, 4, 128, 128, 64, 7, 64),     # one query head per key head, 128-wide heads
+    (16, 1, 32, 48, 17, 3, 0),       # sixteen query heads on one key head, no rotation
+    (8, 4, 72, 80, 0, 0, 8),         # no window
+    (2, 1, 40, 32, 25, 0, 4),        # a window without pooled blocks
+])
+def test_window_attention_ops(dt, tol, H, G, D, V, window, P, dims):
+    outs, caches = window_case(H, G, D, V, window, P, dims, dt)
+    for a, b in zip(caches[DEV], caches["cpu"]):
+        close(a, b, tol)
+    close(outs[DEV][0][:, :H * D], outs["cpu"][0][:, :H * D], tol)       # prepared queries
+    close(outs[DEV][1], outs["cpu"][1], tol * 2)
+
+
+def test_window_attention_matrix_cores_match_plain_kernel():
+    """The same caches through both kernels in bf16 (the plain one is also the fp32 path)."""
+    outs, _ = window_case(8, 2, 64, 64, 40, 12, 32, torch.bfloat16, seed=3)
+    old = sm.WINDOW_MFMA
+    try:
+        sm.WINDOW_MFMA = False
+        plain, _ = window_case(8, 2, 64, 64, 40, 12, 32, torch.bfloat16, seed=3)
+    finally:
+        sm.WINDOW_MFMA = old
+    close(outs[DEV][1], plain[DEV][1], 2e-2)
+
+
+# ----------------------------------------------------------------------------- gated matrix-state recurrences
+@pytest.mark.parametrize("dt,tol", DTYPES)
+@pytest.mark.parametrize("kind,H,D,V", [(sm.SCAN_HGRN2, 3, 20, 28), (sm.SCAN_HGRN2, 2, 64, 128), (sm.SCAN_HGRN2, 1, 100, 5),
+                                        (sm.SCAN_MLSTM, 3, 20, 28), (sm.SCAN_MLSTM, 2, 128, 64), (sm.SCAN_MLSTM, 5, 7, 70)])
+def test_gated_scan(dt, tol, kind, H, D, V):
+    torch.manual_seed(30)
+    cu, pos, slots, _ = batch()
+    if kind == sm.SCAN_HGRN2:
+        parts = (("q", H * D), ("f", H * D), ("v", H * V))
+    else:
+        parts = (("q", H * D), ("k", H * D), ("v", H * V), ("i", H), ("f", H), ("g", H * V))
+    cols, at = {}, 3                                   # parts need not start the row
+    for key, n in parts:
+        cols[key] = at
+        at += n + 1
+    proj = torch.randn(T, at) * 1.5
+    nf = H * D if kind == sm.SCAN_HGRN2 else H
+    fb, ib = torch.randn(nf).to(dt), torch.randn(H).to(dt)
+    lower = torch.rand(H * D).to(dt)
+    normw = torch.randn(V if kind == sm.SCAN_HGRN2 else H * V).to(dt)
+    state = torch.randn(4, H, sm.gated_scan_record(kind, D, V)) * 0.5
+    kw = dict(fbias=fb, ibias=ib if kind == sm.SCAN_MLSTM else None, lower=lower if kind == sm.SCAN_HGRN2 else None,
+              cap=6.0)
+    sc, sg = state.clone(), state.to(DEV).clone()
+    oc = sm.gated_scan(proj, kind, cols, normw, sc, cu, slots, pos, H, D, V, 1e-6, dt, **kw)
+    og = sm.gated_scan(proj.to(DEV), kind, cols, normw.to(DEV), sg, cu.to(DEV), slots.to(DEV), pos.to(DEV), H, D, V,
+                       1e-6, dt, **{k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in kw.items()})
+    close(og, oc, tol)
+    close(sg, sc, 1e-4)
+    assert torch.equal(sg[3].cpu(), state[3]) is False and torch.equal(sg[1].cpu(), state[1])    # the empty sequence's slot
