@@ -149,10 +149,12 @@ int k8s_window_kv_write(void* kcache, void* vcache, void* qkv, long ld, int koff
 int k8s_window_pool(float* kpool, float* vpool, const void* kcache, const void* vcache, const int* block_tables,
                     int max_blocks, const int* tok_seq, const int* positions, int T, int G, int D, int V, int P, int bs,
                     int f32, hipStream_t s);
-int k8s_window_attention(void* out, const void* q, long ldq, const void* gate, long ldg, const void* kcache,
-                         const void* vcache, const float* kpool, const float* vpool, const int* block_tables,
-                         int max_blocks, const int* tok_seq, const int* positions, int T, int H, int G, int D, int V,
-                         int window, int P, float scale, int sink, int bs, int f32, hipStream_t s);
+int k8s_window_tile_rows(int H, int G, int D, int V);
+int k8s_window_attention(void* out, float* pacc, float* pml, const void* q, long ldq, const void* gate, long ldg,
+                         const void* kcache, const void* vcache, const float* kpool, const float* vpool,
+                         const int* block_tables, int max_blocks, const int* tok_seq, const int* positions, int T, int H,
+                         int G, int D, int V, int window, int P, float scale, int sink, int bs, int nsplit, int f32,
+                         hipStream_t s);
 int k8s_window_mfma_ok(int H, int G, int D, int V);
 int k8s_window_attention_mfma(void* out, const void* q, long ldq, const void* gate, long ldg, const void* kcache,
                               const void* vcache, const float* kpool, const float* vpool, const int* block_tables,
@@ -489,13 +491,16 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
     check(k8s_window_pool(P<float>(kpool), P<float>(vpool), P(kcache), P(vcache), P<int>(bt), max_blocks,
                           P<int>(tok_seq), P<int>(positions), T, G, D, V, P_, bs, f32, S(s)), "window_pool");
   });
-  m.def("window_attention", [](uintptr_t out, uintptr_t q, long ldq, uintptr_t gate, long ldg, uintptr_t kcache,
-                               uintptr_t vcache, uintptr_t kpool, uintptr_t vpool, uintptr_t bt, int max_blocks,
-                               uintptr_t tok_seq, uintptr_t positions, int T, int H, int G, int D, int V, int window,
-                               int P_, float scale, int sink, int bs, int f32, int64_t s) {
-    check(k8s_window_attention(P(out), P(q), ldq, P(gate), ldg, P(kcache), P(vcache), P<float>(kpool), P<float>(vpool),
-                               P<int>(bt), max_blocks, P<int>(tok_seq), P<int>(positions), T, H, G, D, V, window, P_,
-                               scale, sink, bs, f32, S(s)), "window_attention");
+  m.def("window_tile_rows", [](int H, int G, int D, int V) { return k8s_window_tile_rows(H, G, D, V); });
+  m.def("window_attention", [](uintptr_t out, uintptr_t pacc, uintptr_t pml, uintptr_t q, long ldq, uintptr_t gate,
+                               long ldg, uintptr_t kcache, uintptr_t vcache, uintptr_t kpool, uintptr_t vpool,
+                               uintptr_t bt, int max_blocks, uintptr_t tok_seq, uintptr_t positions, int T, int H, int G,
+                               int D, int V, int window, int P_, float scale, int sink, int bs, int nsplit, int f32,
+                               int64_t s) {
+    check(k8s_window_attention(P(out), P<float>(pacc), P<float>(pml), P(q), ldq, P(gate), ldg, P(kcache), P(vcache),
+                               P<float>(kpool), P<float>(vpool), P<int>(bt), max_blocks, P<int>(tok_seq),
+                               P<int>(positions), T, H, G, D, V, window, P_, scale, sink, bs, nsplit, f32, S(s)),
+          "window_attention");
   });
   m.def("window_mfma_ok", [](int H, int G, int D, int V) { return k8s_window_mfma_ok(H, G, D, V) != 0; });
   m.def("window_attention_mfma", [](uintptr_t out, uintptr_t q, long ldq, uintptr_t gate, long ldg, uintptr_t kcache,

@@ -122,25 +122,48 @@ __global__ __launch_bounds__(256) void window_pool_kernel(float* __restrict__ kp
   }
 }
 
-// One workgroup per (token, key / value head); one wave per query head of the group (further passes when the group has
-// more heads than waves).  The visible keys are an ordered list: the nb pooled blocks, then the window's tokens.  They
-// come in tiles of KB <= 64 rows staged in LDS as fp32 and shared by the group's heads; lane l scores row l
+// 8 consecutive elements of a cached row as fp32 (one or two 16-byte loads).
+__device__ __forceinline__ void load8(const bf16_t* p, float* o) {
+  const u32x4 v = *reinterpret_cast<const u32x4*>(p);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    o[2 * i] = lo_bf(v[i]);
+    o[2 * i + 1] = hi_bf(v[i]);
+  }
+}
+__device__ __forceinline__ void load8(const float* p, float* o) {
+  const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    o[i] = a[i];
+    o[4 + i] = b[i];
+  }
+}
+
+// One workgroup per (token, key / value head, key split); one wave per query head of the group (further passes when
+// the group has more heads than waves).  The visible keys are an ordered list: the nb pooled blocks, then the window's
+// tokens.  They come in tiles of KB <= 64 rows staged in LDS as fp32 and shared by the group's heads (the rows' cache
+// slots are resolved once per tile; VEC: rows move as 16-byte vectors, D and V multiples of 8); lane l scores row l
 // (q . k * scale), the tile joins a running softmax, lane l accumulates value dimensions l, l + 64, ...
-// A sink starts the running softmax at (max 0, sum 1).  out[t][head][V] = sum p v / sum, times sigmoid(gate) if given.
-template <typename TA, int NACC>
-__global__ void window_attention_kernel(TA* __restrict__ out, const TA* __restrict__ q, long ldq,
-                                        const TA* __restrict__ gate, long ldg, const TA* __restrict__ kcache,
-                                        const TA* __restrict__ vcache, const float* __restrict__ kpool,
-                                        const float* __restrict__ vpool, const int* __restrict__ block_tables,
-                                        int max_blocks, const int* __restrict__ tok_seq,
-                                        const int* __restrict__ positions, int H, int G, int D, int V, int window,
-                                        int P, float scale, int sink, int bs, int ppb, int KB) {
+// A sink starts the running softmax at (max 0, sum 1).  One split: out[t][head][V] = sum p v / sum, times
+// sigmoid(gate) if given.  Several splits (few tokens, many keys: decoding) each take a run of tiles and leave
+// (max, sum, unnormalised sum p v) for window_merge_kernel; the sink belongs to split 0.
+template <typename TA, int NACC, bool VEC>
+__global__ void window_attention_kernel(TA* __restrict__ out, float* __restrict__ pacc, float* __restrict__ pml,
+                                        const TA* __restrict__ q, long ldq, const TA* __restrict__ gate, long ldg,
+                                        const TA* __restrict__ kcache, const TA* __restrict__ vcache,
+                                        const float* __restrict__ kpool, const float* __restrict__ vpool,
+                                        const int* __restrict__ block_tables, int max_blocks,
+                                        const int* __restrict__ tok_seq, const int* __restrict__ positions, int H, int G,
+                                        int D, int V, int window, int P, float scale, int sink, int bs, int ppb, int KB,
+                                        int nsplit) {
   extern __shared__ float smem[];
-  const int t = blockIdx.x, g = blockIdx.y;
+  const int t = blockIdx.x, g = blockIdx.y, split = blockIdx.z;
   const int R = H / G;
   const int p = positions[t];
   if (p < 0) {   // idle row: defined output, nothing read
-    for (int i = threadIdx.x; i < R * V; i += blockDim.x) stf(out, (size_t)t * H * V + (size_t)g * R * V + i, 0.f);
+    if (nsplit == 1)
+      for (int i = threadIdx.x; i < R * V; i += blockDim.x) stf(out, (size_t)t * H * V + (size_t)g * R * V + i, 0.f);
     return;
   }
   const int DP = D + 1;
@@ -148,36 +171,71 @@ __global__ void window_attention_kernel(TA* __restrict__ out, const TA* __restri
   float* ktile = smem;                         // [KB][D + 1]
   float* vtile = ktile + (size_t)KB * DP;      // [KB][V]
   float* qs = vtile + (size_t)KB * V;          // [nw][D]
+  size_t roff = (size_t)KB * (DP + V) + (size_t)nw * D;
+  roff += roff & 1;                            // 8-byte aligned
+  long long* rowoff = reinterpret_cast<long long*>(smem + roff);   // [KB] a tile row's cache slot, or -1 - pool entry
   const int lo = window > 0 ? max(0, p - window + 1) : 0;
   const int nb = (window > 0 && P > 0 && p - window + 1 >= P) ? (p - window + 1) / P : 0;
   const int nkeys = nb + (p + 1 - lo);
+  const int ntiles = (nkeys + KB - 1) / KB;
+  const int tps = (ntiles + nsplit - 1) / nsplit;
+  const int tile0 = split * tps, tile1 = min(ntiles, tile0 + tps);
   const int* btr = block_tables + (size_t)tok_seq[t] * max_blocks;
   const int GD = G * D, GV = G * V;
+  const bool with_sink = sink && split == 0;
   for (int h0 = 0; h0 < R; h0 += nw) {
     const int hd = g * R + h0 + wave;
     const bool hv = h0 + wave < R;
     float* qq = qs + (size_t)wave * D;
     if (hv)
       for (int d = lane; d < D; d += 64) qq[d] = ldf(q, (size_t)t * ldq + (size_t)hd * D + d);
-    float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f, acc[NACC];
+    float m = with_sink ? 0.f : -INFINITY, l = with_sink ? 1.f : 0.f, acc[NACC];
 #pragma unroll
     for (int i = 0; i < NACC; ++i) acc[i] = 0.f;
-    for (int u0 = 0; u0 < nkeys; u0 += KB) {
+    for (int tile = tile0; tile < tile1; ++tile) {
+      const int u0 = tile * KB;
       const int nk = min(KB, nkeys - u0);
       __syncthreads();
-      for (int idx = tid; idx < nk * (D + V); idx += blockDim.x) {
-        const int r = idx / (D + V), d = idx - r * (D + V), u = u0 + r;
-        float val;
+      for (int r = tid; r < nk; r += blockDim.x) {
+        const int u = u0 + r;
         if (u < nb) {
-          const size_t e = pool_entry(btr, u, P, bs, ppb);
-          val = d < D ? kpool[e * GD + (size_t)g * D + d] : vpool[e * GV + (size_t)g * V + (d - D)];
+          rowoff[r] = -1 - (long long)pool_entry(btr, u, P, bs, ppb);
         } else {
           const int j = lo + (u - nb);
-          const size_t slot = (size_t)btr[j / bs] * bs + (j % bs);
-          val = d < D ? ldf(kcache, slot * GD + (size_t)g * D + d) : ldf(vcache, slot * GV + (size_t)g * V + (d - D));
+          rowoff[r] = (long long)btr[j / bs] * bs + (j % bs);
         }
-        if (d < D) ktile[r * DP + d] = val;
-        else vtile[r * V + (d - D)] = val;
+      }
+      __syncthreads();
+      if (VEC) {
+        const int ckd = D >> 3, cpr = ckd + (V >> 3);
+        for (int idx = tid; idx < nk * cpr; idx += blockDim.x) {
+          const int r = idx / cpr, c = idx - r * cpr;
+          const bool isk = c < ckd;
+          const int e8 = 8 * (isk ? c : c - ckd);
+          const long long ro = rowoff[r];
+          float v8[8];
+          if (ro < 0) load8(isk ? kpool + (size_t)(-1 - ro) * GD + (size_t)g * D + e8
+                                : vpool + (size_t)(-1 - ro) * GV + (size_t)g * V + e8, v8);
+          else load8(isk ? kcache + (size_t)ro * GD + (size_t)g * D + e8 : vcache + (size_t)ro * GV + (size_t)g * V + e8, v8);
+          float* dst = isk ? ktile + r * DP + e8 : vtile + r * V + e8;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) dst[i] = v8[i];
+        }
+      } else {
+        for (int idx = tid; idx < nk * (D + V); idx += blockDim.x) {
+          const int r = idx / (D + V), d = idx - r * (D + V);
+          const long long ro = rowoff[r];
+          float val;
+          if (ro < 0) {
+            const size_t e = (size_t)(-1 - ro);
+            val = d < D ? kpool[e * GD + (size_t)g * D + d] : vpool[e * GV + (size_t)g * V + (d - D)];
+          } else {
+            val = d < D ? ldf(kcache, (size_t)ro * GD + (size_t)g * D + d)
+                        : ldf(vcache, (size_t)ro * GV + (size_t)g * V + (d - D));
+          }
+          if (d < D) ktile[r * DP + d] = val;
+          else vtile[r * V + (d - D)] = val;
+        }
       }
       __syncthreads();
       if (hv) {
@@ -205,7 +263,7 @@ __global__ void window_attention_kernel(TA* __restrict__ out, const TA* __restri
         }
       }
     }
-    if (hv) {
+    if (hv && nsplit == 1) {
 #pragma unroll
       for (int i = 0; i < NACC; ++i) {
         const int d = lane + 64 * i;
@@ -215,10 +273,50 @@ __global__ void window_attention_kernel(TA* __restrict__ out, const TA* __restri
           stf(out, (size_t)t * H * V + (size_t)hd * V + d, o);
         }
       }
+    } else if (hv) {
+      const size_t rec = ((size_t)t * H + hd) * nsplit + split;
+#pragma unroll
+      for (int i = 0; i < NACC; ++i) {
+        const int d = lane + 64 * i;
+        if (d < V) pacc[rec * V + d] = acc[i];
+      }
+      if (lane == 0) {
+        pml[rec * 2] = m;           // -inf and 0 for a split without tiles and without the sink
+        pml[rec * 2 + 1] = l;
+      }
     }
   }
 }
 
+// out[t][head] = sum_s e^(m_s - M) acc_s / sum_s e^(m_s - M) l_s over the key splits, times sigmoid(gate) if given.
+template <typename TA>
+__global__ void window_merge_kernel(TA* __restrict__ out, const float* __restrict__ pacc, const float* __restrict__ pml,
+                                    const TA* __restrict__ gate, long ldg, const int* __restrict__ positions, int H,
+                                    int V, int nsplit) {
+  const int t = blockIdx.x, hd = blockIdx.y;
+  if (positions[t] < 0) {
+    for (int d = threadIdx.x; d < V; d += blockDim.x) stf(out, (size_t)t * H * V + (size_t)hd * V + d, 0.f);
+    return;
+  }
+  const size_t rec0 = ((size_t)t * H + hd) * nsplit;
+  float M = -INFINITY;
+  for (int s = 0; s < nsplit; ++s) M = fmaxf(M, pml[(rec0 + s) * 2]);
+  float den = 0.f;
+  for (int s = 0; s < nsplit; ++s) {
+    const float ms = pml[(rec0 + s) * 2];
+    if (ms != -INFINITY) den += expf(ms - M) * pml[(rec0 + s) * 2 + 1];
+  }
+  for (int d = threadIdx.x; d < V; d += blockDim.x) {
+    float a = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+      const float ms = pml[(rec0 + s) * 2];
+      if (ms != -INFINITY) a += expf(ms - M) * pacc[(rec0 + s) * V + d];
+    }
+    float o = a / den;
+    if (gate != nullptr) o *= 1.f / (1.f + expf(-ldf(gate, (size_t)t * ldg + (size_t)hd * V + d)));
+    stf(out, (size_t)t * H * V + (size_t)hd * V + d, o);
+  }
+}
 
 // The same attention on the matrix cores for prompts in bf16 (D % 8 == 0, V % 16 == 0, R = H / G a power of two <= 16).
 // A workgroup of 4 waves takes TPB consecutive tokens of one sequence and one key / value head; a wave owns NCB blocks
@@ -476,37 +574,61 @@ extern "C" int k8s_window_pool(float* kpool, float* vpool, const void* kcache, c
   return (int)hipGetLastError();
 }
 
-extern "C" int k8s_window_attention(void* out, const void* q, long ldq, const void* gate, long ldg, const void* kcache,
-                                    const void* vcache, const float* kpool, const float* vpool,
-                                    const int* block_tables, int max_blocks, const int* tok_seq, const int* positions,
-                                    int T, int H, int G, int D, int V, int window, int P, float scale, int sink, int bs,
-                                    int f32, hipStream_t s) {
+// Tile rows of the plain kernel for these sizes (0: they do not fit) -- the caller sizes the key splits with it.
+extern "C" int k8s_window_tile_rows(int H, int G, int D, int V) {
+  if (G <= 0 || H % G) return 0;
+  const int R = H / G, nw = R < 8 ? R : 8;
+  // LDS floats: KB (D + 1 + V) tile + nw D queries + KB row offsets (2 floats each), within 60 KB
+  int KB = (15360 - nw * D - 2) / (D + 1 + V + 2);
+  return KB > 64 ? 64 : (KB < 1 ? 0 : KB);
+}
+
+// nsplit > 1: pacc [T, H, nsplit, V] and pml [T, H, nsplit, 2] fp32 workspaces.
+extern "C" int k8s_window_attention(void* out, float* pacc, float* pml, const void* q, long ldq, const void* gate,
+                                    long ldg, const void* kcache, const void* vcache, const float* kpool,
+                                    const float* vpool, const int* block_tables, int max_blocks, const int* tok_seq,
+                                    const int* positions, int T, int H, int G, int D, int V, int window, int P,
+                                    float scale, int sink, int bs, int nsplit, int f32, hipStream_t s) {
   if (T <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G || D <= 0 || V <= 0 || V > 256 || bs <= 0 || G > 65535) return -1;
   if (window > 0 && P > 0 && (kpool == nullptr || vpool == nullptr)) return -1;
+  if (nsplit < 1 || nsplit > 65535 || (nsplit > 1 && (pacc == nullptr || pml == nullptr))) return -1;
   const int R = H / G;
   const int nw = R < 8 ? R : 8;
-  // LDS floats: KB (D + 1 + V) tile + nw D queries, within 60 KB
-  int KB = (15360 - nw * D) / (D + 1 + V);
-  if (KB > 64) KB = 64;
+  const int KB = k8s_window_tile_rows(H, G, D, V);
   if (KB < 1) return -2;
-  const size_t lds = ((size_t)KB * (D + 1 + V) + (size_t)nw * D) * sizeof(float);
+  const size_t lds = ((size_t)KB * (D + 1 + V) + (size_t)nw * D + 2 + 2 * (size_t)KB) * sizeof(float);
   const int ppb = P > 0 ? (bs + P - 1) / P : 1;
   const int nacc = (V + 63) / 64;
-#define K8S_WA(TA, NA)                                                                                                \
-  window_attention_kernel<TA, NA><<<dim3(T, G), nw * 64, lds, s>>>(                                                   \
-      (TA*)out, (const TA*)q, ldq, (const TA*)gate, ldg, (const TA*)kcache, (const TA*)vcache, kpool, vpool,          \
-      block_tables, max_blocks, tok_seq, positions, H, G, D, V, window, P, scale, sink, bs, ppb, KB)
-#define K8S_WA_T(TA)                   \
-  do {                                 \
-    if (nacc <= 1) K8S_WA(TA, 1);      \
-    else if (nacc <= 2) K8S_WA(TA, 2); \
-    else K8S_WA(TA, 4);                \
+  const bool vec = D % 8 == 0 && V % 8 == 0 && (f32 || ((long)G * D) % 8 == 0);
+#define K8S_WA(TA, NA, VEC)                                                                                           \
+  window_attention_kernel<TA, NA, VEC><<<dim3(T, G, nsplit), nw * 64, lds, s>>>(                                      \
+      (TA*)out, pacc, pml, (const TA*)q, ldq, (const TA*)gate, ldg, (const TA*)kcache, (const TA*)vcache, kpool,      \
+      vpool, block_tables, max_blocks, tok_seq, positions, H, G, D, V, window, P, scale, sink, bs, ppb, KB, nsplit)
+#define K8S_WA_V(TA, NA)            \
+  do {                              \
+    if (vec) K8S_WA(TA, NA, true);  \
+    else K8S_WA(TA, NA, false);     \
+  } while (0)
+#define K8S_WA_T(TA)                     \
+  do {                                   \
+    if (nacc <= 1) K8S_WA_V(TA, 1);      \
+    else if (nacc <= 2) K8S_WA_V(TA, 2); \
+    else K8S_WA_V(TA, 4);                \
   } while (0)
   if (f32) K8S_WA_T(float);
   else K8S_WA_T(bf16_t);
 #undef K8S_WA_T
+#undef K8S_WA_V
 #undef K8S_WA
+  if (nsplit > 1) {
+    if (f32)
+      window_merge_kernel<float><<<dim3(T, H), 64, 0, s>>>((float*)out, pacc, pml, (const float*)gate, ldg, positions, H,
+                                                           V, nsplit);
+    else
+      window_merge_kernel<bf16_t><<<dim3(T, H), 64, 0, s>>>((bf16_t*)out, pacc, pml, (const bf16_t*)gate, ldg,
+                                                            positions, H, V, nsplit);
+  }
   return (int)hipGetLastError();
 }
 

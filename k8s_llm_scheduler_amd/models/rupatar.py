@@ -444,7 +444,7 @@ class RupatarModel(StreamModel):
             sm.window_pool(kp, vp, kc, vc, b["block_tables"], b["tok_seq"], b["positions"], m.pool, self.block_size)
         a = sm.window_attention(proj, proj[:, w.goff:w.goff + H * V], kc, vc, kp, vp, b["block_tables"], b["tok_seq"],
                                 b["positions"], H, m.window, m.pool, m.scale, True, self.block_size, b["cu_q"],
-                                b.get("max_qlen", 0))
+                                b.get("max_qlen", 0), b.get("max_keys", 0))
         return sm.linear(a, w.o), w.ob
 
     def _scan(self, w: _Scan, L: _Layer, h, b):

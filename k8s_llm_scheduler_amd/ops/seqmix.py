@@ -429,10 +429,21 @@ def window_pool(kpool: torch.Tensor, vpool: torch.Tensor, kcache: torch.Tensor, 
 WINDOW_MFMA = os.environ.get("K8S_WINDOW_MFMA", "1") != "0"   # 0: always the plain-FMA attention kernel
 
 
+def window_splits(T: int, G: int, window: int, P: int, max_pos: int, tile_rows: int) -> int:
+    """Key splits of the plain windowed attention: one when the (token, key head) grid fills the chip by itself, else
+    enough splits of at least one tile each for about 256 workgroups.  ``max_pos``: positions a token can have."""
+    groups = T * G
+    if groups >= 128 or tile_rows <= 0:
+        return 1
+    keys = max_pos if window <= 0 else min(max_pos, window + (max_pos // P if P > 0 else 0))
+    return max(1, min(256 // groups, -(-max(1, keys) // tile_rows), 16))
+
+
 def window_attention(q: torch.Tensor, gate: Optional[torch.Tensor], kcache: torch.Tensor, vcache: torch.Tensor,
                      kpool: Optional[torch.Tensor], vpool: Optional[torch.Tensor], block_tables: torch.Tensor,
                      tok_seq: torch.Tensor, positions: torch.Tensor, H: int, window: int, P: int, scale: float,
-                     sink: bool, block_size: int, cu_q: Optional[torch.Tensor] = None, max_qlen: int = 0) -> torch.Tensor:
+                     sink: bool, block_size: int, cu_q: Optional[torch.Tensor] = None, max_qlen: int = 0,
+                     max_keys: int = 0) -> torch.Tensor:
     """Grouped-query attention over the paged caches [slots, G, D] / [slots, G, V]: the token at position p sees the
     tokens max(0, p - window + 1) .. p (``window`` <= 0: all) and, with ``P`` > 0, the pooled blocks that lie wholly
     before the window (b P + P - 1 <= p - window), all in one softmax; ``sink``: one more unit in the denominator.
@@ -440,7 +451,8 @@ def window_attention(q: torch.Tensor, gate: Optional[torch.Tensor], kcache: torc
     multiplied by sigmoid(gate).  Returns [T, H V].
     ``cu_q`` / ``max_qlen`` (the sequences' query offsets and longest portion): bf16 portions of prompts whose sizes
     fit run on the matrix cores, tiles of consecutive tokens sharing the staged keys; anything else (fp32, single
-    tokens, other sizes) on the plain-FMA kernel."""
+    tokens, other sizes) on the plain-FMA kernel, which splits the keys of few tokens over several workgroups
+    (``max_keys``: an upper bound of the positions any token sees, 0: the block tables' capacity)."""
     G, D, V = kcache.shape[1], kcache.shape[2], vcache.shape[2]
     if H % G:
         raise ValueError(f"window_attention: {H} query heads over {G} key heads")
@@ -464,12 +476,17 @@ def window_attention(q: torch.Tensor, gate: Optional[torch.Tensor], kcache: torc
                                   _p(positions, I32), cu_q.shape[0] - 1, int(max_qlen), H, G, D, V, int(window), int(P),
                                   float(scale), int(bool(sink)), block_size, -1)
         return out
-    _native().window_attention(out.data_ptr(), q.data_ptr(), q.stride(0), gate.data_ptr() if gate is not None else 0,
-                               gate.stride(0) if gate is not None else 0, _p(kcache, dt, "kcache"),
-                               _p(vcache, dt, "vcache"), _p(kpool, F32, "kpool"), _p(vpool, F32, "vpool"),
-                               _p(block_tables, I32, "block_tables"), block_tables.shape[1], _p(tok_seq, I32),
-                               _p(positions, I32), T, H, G, D, V, int(window), int(P), float(scale), int(bool(sink)),
-                               block_size, _f32(dt), -1)
+    ns = window_splits(T, G, window, P, max_keys or block_tables.shape[1] * block_size, nat.window_tile_rows(H, G, D, V))
+    pacc = pml = None
+    if ns > 1:
+        pacc = torch.empty(T * H * ns * V, dtype=F32, device=q.device)
+        pml = torch.empty(T * H * ns * 2, dtype=F32, device=q.device)
+    nat.window_attention(out.data_ptr(), _p(pacc), _p(pml), q.data_ptr(), q.stride(0),
+                         gate.data_ptr() if gate is not None else 0, gate.stride(0) if gate is not None else 0,
+                         _p(kcache, dt, "kcache"), _p(vcache, dt, "vcache"), _p(kpool, F32, "kpool"),
+                         _p(vpool, F32, "vpool"), _p(block_tables, I32, "block_tables"), block_tables.shape[1],
+                         _p(tok_seq, I32), _p(positions, I32), T, H, G, D, V, int(window), int(P), float(scale),
+                         int(bool(sink)), block_size, ns, _f32(dt), -1)
     return out
 
 
