@@ -165,7 +165,8 @@ long long k8s_gated_scan_record(int kind, int D, int V);
 int k8s_gated_scan(void* out, const float* proj, long ld, int kind, int cq, int ck, int cv, int ci, int cf, int cg,
                    const void* fbias, const void* ibias, const void* lower, const void* normw, float* state,
                    const int* cu_q, const int* seq_slots, const int* positions, int nseq, int H, int D, int V, float eps,
-                   float cap, int f32, hipStream_t s);
+                   float cap, int f32, int T, int Lc, float* ws, hipStream_t s);
+long long k8s_gated_scan_workspace(int T, int nseq, int H, int D, int V, int Lc);
 int k8s_moe_align(int* sorted_tok, int* pos_of_pair, int* seg, int* tiles, int ntiles, const int* topk_idx, int P,
                   int top, int E, int BM, hipStream_t s);
 int k8s_moe_combine(void* z, const void* D, const int* pos, const float* w, const void* shared, const float* logits,
@@ -516,10 +517,13 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
   m.def("gated_scan", [](uintptr_t out, uintptr_t proj, long ld, int kind, int cq, int ck, int cv, int ci, int cf,
                          int cg, uintptr_t fbias, uintptr_t ibias, uintptr_t lower, uintptr_t normw, uintptr_t state,
                          uintptr_t cu_q, uintptr_t seq_slots, uintptr_t positions, int nseq, int H, int D, int V,
-                         float eps, float cap, int f32, int64_t s) {
+                         float eps, float cap, int f32, int T, int Lc, uintptr_t ws, int64_t s) {
     check(k8s_gated_scan(P(out), P<float>(proj), ld, kind, cq, ck, cv, ci, cf, cg, P(fbias), P(ibias), P(lower),
                          P(normw), P<float>(state), P<int>(cu_q), P<int>(seq_slots), P<int>(positions), nseq, H, D, V,
-                         eps, cap, f32, S(s)), "gated_scan");
+                         eps, cap, f32, T, Lc, P<float>(ws), S(s)), "gated_scan");
+  });
+  m.def("gated_scan_workspace", [](int T, int nseq, int H, int D, int V, int Lc) {
+    return k8s_gated_scan_workspace(T, nseq, H, D, V, Lc);
   });
   m.def("moe_align", [](uintptr_t sorted_tok, uintptr_t pos, uintptr_t seg, uintptr_t tiles, int ntiles,
                         uintptr_t topk_idx, int P_, int top, int E, int BM, int64_t s) {

@@ -105,6 +105,19 @@ __device__ __forceinline__ void lds_barrier() {
   asm volatile("" ::: "memory");
 }
 
+// Chunk g of a varlen batch cut into chunks of Lc tokens per sequence: (sequence, chunk in the sequence, chunks of the
+// sequence), or sequence -1 when g is past the last chunk.  Idle (position < 0) and empty sequences have no chunks.
+struct WkvChunk { int s, c, n; };
+__device__ __forceinline__ WkvChunk wkv_find_chunk(int g, const int* cu_q, const int* positions, int nseq, int Lc) {
+  for (int s = 0; s < nseq; ++s) {
+    const int a = cu_q[s], len = cu_q[s + 1] - a;
+    const int n = (len > 0 && positions[a] >= 0) ? (len + Lc - 1) / Lc : 0;
+    if (g < n) return WkvChunk{s, g, n};
+    g -= n;
+  }
+  return WkvChunk{-1, 0, 0};
+}
+
 // 32-bit mixing hash (murmur3 finalizer) used for counter-based RNG and deterministic init.
 __device__ __forceinline__ uint32_t fmix32(uint32_t h) {
   h ^= h >> 16; h *= 0x85ebca6bu; h ^= h >> 13; h *= 0xc2b2ae35u; h ^= h >> 16;

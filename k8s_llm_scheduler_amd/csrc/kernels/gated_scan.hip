@@ -17,12 +17,23 @@ namespace k8sllm {
 
 struct ScanCols { int q, k, v, i, f, g; };   // column offsets of the parts inside a projected row
 
-// One workgroup per (sequence, head).  Thread (x, c) owns value column x of the CH key channels [c CH, (c + 1) CH) of S;
-// group c = 0 prepares each token's per-channel read / keep / write coefficients in LDS (and, KIND 1, owns n).  The
-// partial outputs of the channel groups meet in LDS; group 0 normalises and stores.  The next token's inputs are
-// loaded while the current one is computed; the barriers wait for LDS traffic only.
+// One workgroup per (sequence or chunk, head).  Thread (x, c) owns value column x of the CH key channels
+// [c CH, (c + 1) CH) of S; group c = 0 prepares each token's per-channel read / keep / write coefficients in LDS (and,
+// KIND 1, owns n).  The partial outputs of the channel groups meet in LDS; group 0 normalises and stores.  The next
+// token's inputs are loaded while the current one is computed; the barriers wait for LDS traffic only.
 // blockDim = (DX, NS): DX = max(D, V) rounded up to 64, NS = ceil(D / CH).  State record: S [D][V] (, n [D], m).
-template <typename TA, int CH, int KIND>
+//
+// MODE 0: a whole portion per workgroup, from the slot's state (zero at position 0) to the slot's state.
+// Long portions run as three passes over chunks of Lc tokens, so the recurrence is parallel over chunks; a chunk record
+// is S [D][V], then D floats (KIND 0: the product of the chunk's decays per channel; KIND 1: n), then (KIND 1) m and
+// the sum F of the chunk's log forget gates:
+// MODE 1: a chunk from the empty state, no outputs -> its record in cs_loc (KIND 1: the running maximum starts at
+//         minus infinity, so the record is the chunk's own contribution under its own maximum);
+//         gated_prefix_kernel then walks a sequence's chunks:
+//           KIND 0: start[c + 1] = dec[c] * start[c] + loc[c]
+//           KIND 1: m' = max(F + m, m_loc); (S, n)[c + 1] = e^(F + m - m') (S, n)[c] + e^(m_loc - m') (S, n)_loc
+// MODE 2: a chunk from its start state with outputs; a sequence's last chunk leaves the slot's state.
+template <typename TA, int CH, int KIND, int MODE>
 __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, const float* __restrict__ proj, long ld,
                                                           ScanCols co, const TA* __restrict__ fbias,
                                                           const TA* __restrict__ ibias, const TA* __restrict__ lower,
@@ -30,29 +41,54 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
                                                           const int* __restrict__ cu_q,
                                                           const int* __restrict__ seq_slots,
                                                           const int* __restrict__ positions, int H, int D, int V,
-                                                          float eps, float cap) {
+                                                          float eps, float cap, int nseq, int Lc,
+                                                          float* __restrict__ cs_loc,
+                                                          const float* __restrict__ cs_start) {
   constexpr int DMAX = 128;
   __shared__ __attribute__((aligned(16))) float sq[DMAX], sa[DMAX], sb[DMAX];
   __shared__ float po[DMAX / CH][DMAX];
   __shared__ float red[2], rednq[2];
-  const int s = blockIdx.x, hd = blockIdx.y;
-  const int a0 = cu_q[s], b0 = cu_q[s + 1];
-  if (b0 <= a0) return;
-  const int p0 = positions[a0];
-  if (p0 < 0) return;
-  const bool from_zero = p0 == 0;
+  const int hd = blockIdx.y;
+  int s, a0, b0, p0;
+  bool from_zero, last = true;
+  if (MODE == 0) {
+    s = blockIdx.x;
+    a0 = cu_q[s];
+    b0 = cu_q[s + 1];
+    if (b0 <= a0) return;
+    p0 = positions[a0];
+    if (p0 < 0) return;
+    from_zero = p0 == 0;
+  } else {
+    const WkvChunk ck = wkv_find_chunk(blockIdx.x, cu_q, positions, nseq, Lc);
+    if (ck.s < 0) return;
+    s = ck.s;
+    last = ck.c == ck.n - 1;
+    if (MODE == 1 && last) return;          // nothing follows a sequence's last chunk
+    a0 = cu_q[s] + ck.c * Lc;
+    b0 = min(cu_q[s + 1], a0 + Lc);
+    p0 = positions[a0];
+    from_zero = MODE == 1 || p0 == 0;
+  }
   const int x = threadIdx.x, c = threadIdx.y, NS = blockDim.y, DX = blockDim.x;
   const bool onv = x < V, ond = x < D;
   const int i0 = c * CH;
-  const size_t rec = (size_t)D * V + (KIND == 1 ? D + 1 : 0);
+  const size_t rec = (size_t)D * V + (KIND == 1 ? D + 1 : 0);       // slot record
+  const size_t crec = (size_t)D * V + D + 2;                         // chunk record
   float* st = state + ((size_t)seq_slots[s] * H + hd) * rec;
-  float S[CH];
+  const size_t cbase = ((size_t)blockIdx.x * H + hd) * crec;         // this chunk's record in cs_loc / cs_start
+  // MODE 2 never reads the slot's record, which the sequence's last chunk overwrites: the prefix pass left a copy
+  const float* src = MODE == 2 ? cs_start + cbase : st;
+  float S[CH], decp[CH];
 #pragma unroll
-  for (int e = 0; e < CH; ++e) S[e] = (onv && i0 + e < D && !from_zero) ? st[(size_t)(i0 + e) * V + x] : 0.f;
-  float nx = 0.f, m = 0.f;
+  for (int e = 0; e < CH; ++e) {
+    S[e] = (onv && i0 + e < D && !from_zero) ? src[(size_t)(i0 + e) * V + x] : 0.f;
+    decp[e] = 1.f;
+  }
+  float nx = 0.f, m = MODE == 1 ? -INFINITY : 0.f, fsum = 0.f;
   if (KIND == 1 && !from_zero) {
-    if (c == 0 && ond) nx = st[(size_t)D * V + x];
-    m = st[(size_t)D * V + D];
+    if (c == 0 && ond) nx = src[(size_t)D * V + x];
+    m = src[(size_t)D * V + D];
   }
   if (c == 0)
     for (int e = x; e < DMAX; e += DX) sq[e] = sa[e] = sb[e] = 0.f;
@@ -62,11 +98,11 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
       lowx = ldf(lower, (size_t)hd * D + x);
       fbx = fbias != nullptr ? ldf(fbias, (size_t)hd * D + x) : 0.f;
     }
-    if (c == 0 && onv) nwx = ldf(normw, x);
+    if (MODE != 1 && c == 0 && onv) nwx = ldf(normw, x);
   } else {
     fbh = fbias != nullptr ? ldf(fbias, hd) : 0.f;
     ibh = ibias != nullptr ? ldf(ibias, hd) : 0.f;
-    if (c == 0 && onv) nwx = ldf(normw, (size_t)hd * V + x);
+    if (MODE != 1 && c == 0 && onv) nwx = ldf(normw, (size_t)hd * V + x);
   }
   const float qscale = KIND == 1 ? 1.0f / sqrtf((float)D) : 1.f;
   lds_barrier();
@@ -79,10 +115,10 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
     if (KIND == 1) {
       nf = r[co.f + hd];
       ni = r[co.i + hd];
-      if (c == 0 && onv) ng = r[co.g + (size_t)hd * V + x];
+      if (MODE != 1 && c == 0 && onv) ng = r[co.g + (size_t)hd * V + x];
     }
     if (c == 0 && ond) {
-      nq = r[co.q + (size_t)hd * D + x];
+      if (MODE != 1) nq = r[co.q + (size_t)hd * D + x];
       if (KIND == 0) nf = r[co.f + (size_t)hd * D + x];
       else nk = r[co.k + (size_t)hd * D + x];
     }
@@ -104,9 +140,10 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
       const float fr = cap * tanhf((cf + fbh) / cap);
       const float fg = fminf(fr, 0.f) - log1pf(expf(-fabsf(fr)));
       const float mn = fmaxf(fg + m, ig);
-      ka = expf(fg + m - mn);
+      ka = expf(fg + m - mn);           // 0 at the first token of a chunk from the empty state (m = -inf)
       const float kb = expf(ig - mn);
       m = mn;
+      fsum += fg;
       if (c == 0) {
         float nqp = 0.f;
         if (ond) {
@@ -116,8 +153,10 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
           sq[x] = qv;
           sb[x] = kb * ck;
         }
-        nqp = wave_sum(nqp);
-        if ((x & 63) == 0) rednq[x >> 6] = nqp;
+        if (MODE != 1) {
+          nqp = wave_sum(nqp);
+          if ((x & 63) == 0) rednq[x >> 6] = nqp;
+        }
       }
     }
     lds_barrier();
@@ -131,8 +170,13 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         S[e0 + e] = fmaf(a4[e], S[e0 + e], b4[e] * cv);
-        o4[e] = fmaf(q4[e], S[e0 + e], o4[e]);
+        if (MODE != 1) o4[e] = fmaf(q4[e], S[e0 + e], o4[e]);
+        if (MODE == 1 && KIND == 0) decp[e0 + e] *= a4[e];
       }
+    }
+    if (MODE == 1) {
+      lds_barrier();                   // the LDS rows are free for the next token
+      continue;
     }
     if (onv) po[c][x] = (o4[0] + o4[1]) + (o4[2] + o4[3]);
     lds_barrier();
@@ -157,14 +201,72 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
       stf(out, (size_t)t * H * V + (size_t)hd * V + x, y);
     }
   }
+  if (MODE == 2 && !last) return;
+  float* dst = MODE == 1 ? cs_loc + cbase : st;
   if (onv) {
 #pragma unroll
     for (int e = 0; e < CH; ++e)
-      if (i0 + e < D) st[(size_t)(i0 + e) * V + x] = S[e];
+      if (i0 + e < D) dst[(size_t)(i0 + e) * V + x] = S[e];
   }
   if (KIND == 1 && c == 0) {
-    if (ond) st[(size_t)D * V + x] = nx;
-    if (x == 0) st[(size_t)D * V + D] = m;
+    if (ond) dst[(size_t)D * V + x] = nx;
+    if (x == 0) {
+      dst[(size_t)D * V + D] = m;
+      if (MODE == 1) dst[(size_t)D * V + D + 1] = fsum;
+    }
+  }
+  if (KIND == 0 && MODE == 1 && x == 0) {
+#pragma unroll
+    for (int e = 0; e < CH; ++e)
+      if (i0 + e < D) dst[(size_t)D * V + i0 + e] = decp[e];
+  }
+}
+
+// Start states of a sequence's chunks from the slot's state (zero at position 0: chunk 0 has no record then) and the
+// chunks' records.
+// One workgroup per (sequence, head); every thread walks the chunks for its elements of (S, n).
+template <int KIND>
+__global__ void gated_prefix_kernel(float* __restrict__ cs_start, const float* __restrict__ cs_loc,
+                                    const float* __restrict__ state, const int* __restrict__ cu_q,
+                                    const int* __restrict__ seq_slots, const int* __restrict__ positions, int H, int D,
+                                    int V, int Lc) {
+  const int s = blockIdx.x, hd = blockIdx.y;
+  int first = 0;
+  for (int y = 0; y < s; ++y) {
+    const int a = cu_q[y], len = cu_q[y + 1] - a;
+    first += (len > 0 && positions[a] >= 0) ? (len + Lc - 1) / Lc : 0;
+  }
+  const int a = cu_q[s], len = cu_q[s + 1] - a;
+  if (len <= 0 || positions[a] < 0) return;
+  const int n = (len + Lc - 1) / Lc;
+  const bool zero = positions[a] == 0;
+  if (zero && n < 2) return;
+  const int DV = D * V;
+  const size_t rec = (size_t)DV + (KIND == 1 ? D + 1 : 0), crec = (size_t)DV + D + 2;
+  const float* st = state + ((size_t)seq_slots[s] * H + hd) * rec;
+  const int nel = KIND == 1 ? DV + D : DV;
+  float* own = cs_start + ((size_t)first * H + hd) * crec;        // chunk 0 starts from a copy of the slot's record
+  for (int e = threadIdx.x; e < nel; e += blockDim.x) {
+    float X = zero ? 0.f : st[e];
+    float m = (KIND == 1 && !zero) ? st[DV + D] : 0.f;
+    if (!zero) {
+      own[e] = X;
+      if (KIND == 1 && e == 0) own[DV + D] = m;
+    }
+    for (int c = 0; c + 1 < n; ++c) {
+      const float* loc = cs_loc + ((size_t)(first + c) * H + hd) * crec;
+      float* nxt = cs_start + ((size_t)(first + c + 1) * H + hd) * crec;
+      if (KIND == 0) {
+        X = fmaf(loc[DV + e / V], X, loc[e]);
+      } else {
+        const float ml = loc[DV + D], F = loc[DV + D + 1];
+        const float mn = fmaxf(F + m, ml);
+        X = expf(F + m - mn) * X + expf(ml - mn) * loc[e];
+        m = mn;
+        if (e == 0) nxt[DV + D] = m;
+      }
+      nxt[e] = X;
+    }
   }
 }
 
@@ -179,10 +281,18 @@ extern "C" long long k8s_gated_scan_record(int kind, int D, int V) {
   return (long long)D * V + (kind == 1 ? D + 1 : 0);
 }
 
+// ws (chunked passes): floats for 2 x chunks x H chunk records, chunks = ceil(T / Lc) + nseq; Lc == 0 (or no
+// workspace): one workgroup per sequence.
+extern "C" long long k8s_gated_scan_workspace(int T, int nseq, int H, int D, int V, int Lc) {
+  if (Lc <= 0) return 0;
+  const long long chunks = (T + Lc - 1) / Lc + nseq;
+  return 2 * chunks * H * ((long long)D * V + D + 2);
+}
+
 extern "C" int k8s_gated_scan(void* out, const float* proj, long ld, int kind, int cq, int ck, int cv, int ci, int cf,
                               int cg, const void* fbias, const void* ibias, const void* lower, const void* normw,
                               float* state, const int* cu_q, const int* seq_slots, const int* positions, int nseq, int H,
-                              int D, int V, float eps, float cap, int f32, hipStream_t s) {
+                              int D, int V, float eps, float cap, int f32, int T, int Lc, float* ws, hipStream_t s) {
   if (nseq <= 0) return 0;
   if (H <= 0 || H > 65535 || D <= 0 || D > 128 || V <= 0 || V > 128 || kind < 0 || kind > 1) return -1;
   if (kind == 0 && lower == nullptr) return -1;
@@ -191,18 +301,35 @@ extern "C" int k8s_gated_scan(void* out, const float* proj, long ld, int kind, i
   const int m = D > V ? D : V;
   const dim3 block((m + 63) / 64 * 64, (D + CH - 1) / CH);
   const ScanCols co{cq, ck, cv, ci, cf, cg};
-#define K8S_GS(TA, KIND)                                                                                            \
-  gated_scan_kernel<TA, CH, KIND><<<dim3(nseq, H), block, 0, s>>>((TA*)out, proj, ld, co, (const TA*)fbias,          \
-                                                                  (const TA*)ibias, (const TA*)lower,               \
-                                                                  (const TA*)normw, state, cu_q, seq_slots,         \
-                                                                  positions, H, D, V, eps, cap)
-  if (kind == 0) {
-    if (f32) K8S_GS(float, 0);
-    else K8S_GS(bf16_t, 0);
-  } else {
-    if (f32) K8S_GS(float, 1);
-    else K8S_GS(bf16_t, 1);
+#define K8S_GS(TA, KIND, MODE, GX, LOC, START)                                                                      \
+  gated_scan_kernel<TA, CH, KIND, MODE><<<dim3(GX, H), block, 0, s>>>(                                              \
+      (TA*)out, proj, ld, co, (const TA*)fbias, (const TA*)ibias, (const TA*)lower, (const TA*)normw, state, cu_q,  \
+      seq_slots, positions, H, D, V, eps, cap, nseq, Lc, LOC, START)
+#define K8S_GS_K(TA, MODE, GX, LOC, START)                  \
+  do {                                                      \
+    if (kind == 0) K8S_GS(TA, 0, MODE, GX, LOC, START);     \
+    else K8S_GS(TA, 1, MODE, GX, LOC, START);               \
+  } while (0)
+#define K8S_GS_T(MODE, GX, LOC, START)                      \
+  do {                                                      \
+    if (f32) K8S_GS_K(float, MODE, GX, LOC, START);         \
+    else K8S_GS_K(bf16_t, MODE, GX, LOC, START);            \
+  } while (0)
+  if (Lc <= 0 || ws == nullptr) {
+    K8S_GS_T(0, nseq, nullptr, nullptr);
+    return (int)hipGetLastError();
   }
+  const int chunks = (T + Lc - 1) / Lc + nseq;
+  float* loc = ws;
+  float* start = ws + (size_t)chunks * H * ((size_t)D * V + D + 2);
+  K8S_GS_T(1, chunks, loc, nullptr);
+  if (kind == 0)
+    gated_prefix_kernel<0><<<dim3(nseq, H), 256, 0, s>>>(start, loc, state, cu_q, seq_slots, positions, H, D, V, Lc);
+  else
+    gated_prefix_kernel<1><<<dim3(nseq, H), 256, 0, s>>>(start, loc, state, cu_q, seq_slots, positions, H, D, V, Lc);
+  K8S_GS_T(2, chunks, nullptr, start);
+#undef K8S_GS_T
+#undef K8S_GS_K
 #undef K8S_GS
   return (int)hipGetLastError();
 }

@@ -41,19 +41,6 @@ __global__ void shift_save_kernel(TA* __restrict__ state, const TA* __restrict__
   for (int i = threadIdx.x; i < W; i += blockDim.x) state[dst + i] = h[src + i];
 }
 
-// Chunk g of a varlen batch cut into chunks of Lc tokens per sequence: (sequence, chunk in the sequence, chunks of the
-// sequence), or sequence -1 when g is past the last chunk.  Idle (position < 0) and empty sequences have no chunks.
-struct WkvChunk { int s, c, n; };
-__device__ __forceinline__ WkvChunk wkv_find_chunk(int g, const int* cu_q, const int* positions, int nseq, int Lc) {
-  for (int s = 0; s < nseq; ++s) {
-    const int a = cu_q[s], len = cu_q[s + 1] - a;
-    const int n = (len > 0 && positions[a] >= 0) ? (len + Lc - 1) / Lc : 0;
-    if (g < n) return WkvChunk{s, g, n};
-    g -= n;
-  }
-  return WkvChunk{-1, 0, 0};
-}
-
 // One workgroup per (sequence or chunk, head).  The head's state S[i][j] (i: key channel, j: value channel) lives in
 // registers: thread (j, c) owns column j of the CH key channels [c CH, (c + 1) CH), so the per-token chain of a wave is
 // CH steps, not D.  Per token:  o_j = sum_i r_i (S_ij + u_i k_i v_j);  S_ij = w_i S_ij + k_i v_j  with

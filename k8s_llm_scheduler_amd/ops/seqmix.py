@@ -500,10 +500,16 @@ def gated_scan_record(kind: int, D: int, V: int) -> int:
     return ref.gated_scan_record(kind, D, V)
 
 
+# Batches of at least SCAN_CHUNK_MIN tokens run the recurrences as three passes over chunks of SCAN_CHUNK tokens (parallel
+# over chunks); shorter ones (decoding, short portions) as one workgroup per sequence.
+SCAN_CHUNK = int(os.environ.get("K8S_SCAN_CHUNK", "64"))
+SCAN_CHUNK_MIN = int(os.environ.get("K8S_SCAN_CHUNK_MIN", "256"))
+
+
 def gated_scan(proj: torch.Tensor, kind: int, cols: dict, normw: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor,
                seq_slots: torch.Tensor, positions: torch.Tensor, H: int, D: int, V: int, eps: float, out_dtype, *,
                fbias: Optional[torch.Tensor] = None, ibias: Optional[torch.Tensor] = None,
-               lower: Optional[torch.Tensor] = None, cap: float = 0.0) -> torch.Tensor:
+               lower: Optional[torch.Tensor] = None, cap: float = 0.0, chunk: Optional[int] = None) -> torch.Tensor:
     """A gated linear recurrence with a matrix state per head over a varlen batch; ``proj`` fp32 [T, ld] is the fused
     input projection with its parts at the column offsets ``cols``; ``state`` [slots, H, record] fp32 is updated in
     place (a portion at position 0 starts from zero).  Returns the normed (and, SCAN_MLSTM, gated) outputs [T, H V].
@@ -528,8 +534,12 @@ def gated_scan(proj: torch.Tensor, kind: int, cols: dict, normw: torch.Tensor, s
     T = proj.shape[0]
     out = torch.empty(T, H * V, dtype=out_dtype, device=proj.device)
     c = lambda key: int(cols.get(key, 0))
+    nseq = cu_q.shape[0] - 1
+    Lc = (SCAN_CHUNK if T >= SCAN_CHUNK_MIN else 0) if chunk is None else int(chunk)
+    ws = torch.empty(_native().gated_scan_workspace(T, nseq, H, D, V, Lc), dtype=F32, device=proj.device) if Lc > 0 \
+        else None
     _native().gated_scan(out.data_ptr(), _p(proj), proj.stride(0), kind, c("q"), c("k"), c("v"), c("i"), c("f"), c("g"),
                          _p(fbias, out_dtype, "fbias"), _p(ibias, out_dtype, "ibias"), _p(lower, out_dtype, "lower"),
                          _p(normw, out_dtype, "normw"), _p(state), _p(cu_q, I32), _p(seq_slots, I32),
-                         _p(positions, I32), cu_q.shape[0] - 1, H, D, V, float(eps), float(cap), _f32(out_dtype), -1)
+                         _p(positions, I32), nseq, H, D, V, float(eps), float(cap), _f32(out_dtype), T, Lc, _p(ws), -1)
     return out

@@ -371,3 +371,9 @@ def test_gated_scan(dt, tol, kind, H, D, V):
     close(og, oc, tol)
     close(sg, sc, 1e-4)
     assert torch.equal(sg[3].cpu(), state[3]) is False and torch.equal(sg[1].cpu(), state[1])    # the empty sequence's slot
+    for chunk in (4, 7, 16, 64):                       # three passes over chunks: same outputs, same final states
+        s2 = state.to(DEV).clone()
+        o2 = sm.gated_scan(proj.to(DEV), kind, cols, normw.to(DEV), s2, cu.to(DEV), slots.to(DEV), pos.to(DEV), H, D, V,
+                           1e-6, dt, chunk=chunk, **{k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in kw.items()})
+        close(o2, oc, tol)
+        close(s2, sc, 1e-4)
