@@ -8,6 +8,10 @@ or any header is newer.  Cross-compiles without a GPU.
 
     python -m k8s_llm_scheduler_amd._build [-j N] [--force] [-v] [--checked]
 
+``--lean`` builds ``ops/_C_lean*.so`` (``-DK8S_LEAN``, objects under ``build/native_lean``): the runtime, the sampler and
+the kernels of the fp32-stream model designs only -- what a fresh checkout compiles before it replays a trace of such a
+model; it is loaded when the full module is absent, and every matrix product then runs on the any-shape GEMM.
+
 ``--checked`` builds the bounds-checked variant ``ops/_C_checked*.so`` (``-DK8S_CHECKED``, objects under
 ``build/native_checked``; loaded instead of ``_C`` when ``K8S_CHECKED=1``): kernels range-check every index they
 derive from data and record violations for the host (csrc/kernels/common.h).
@@ -34,10 +38,14 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # the option on every file, the two-rank fused GEMV all-reduce check of tests/test_multigpu.py reported a wrong sum.
 NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 NO_PACKED_FP32_FILES = {"stream32.hip", "mixers.hip", "moe.hip", "window_attn.hip", "gated_scan.hip"}
+# the lean module: kernels of the fp32-stream designs, the sampler, the small shared kernels; the block allocator
+LEAN_KERNELS = NO_PACKED_FP32_FILES | {"sampler.hip", "misc.hip", "norm.hip"}
+LEAN_RUNTIME = {"block_allocator.cpp"}
 
 
-def ext_path(checked: bool = False) -> Path:
-    return PKG / "ops" / (("_C_checked" if checked else "_C") + sysconfig.get_config_var("EXT_SUFFIX"))
+def ext_path(checked: bool = False, lean: bool = False) -> Path:
+    name = "_C_lean" if lean else "_C_checked" if checked else "_C"
+    return PKG / "ops" / (name + sysconfig.get_config_var("EXT_SUFFIX"))
 
 
 def _torch_dirs():
@@ -66,22 +74,30 @@ def _run(cmd: List[str], verbose: bool) -> None:
         raise RuntimeError(f"command failed ({r.returncode}): {' '.join(cmd)}\n{r.stdout}\n{r.stderr}")
 
 
-def build(jobs: int = 0, force: bool = False, verbose: bool = False, checked: bool = False) -> Path:
+def build(jobs: int = 0, force: bool = False, verbose: bool = False, checked: bool = False, lean: bool = False) -> Path:
     import pybind11
 
+    if checked and lean:
+        raise ValueError("the lean module has no checked variant")
     tinc, tlib, cxx11 = _torch_dirs()
-    bdir = BUILD.parent / "native_checked" if checked else BUILD
+    bdir = BUILD.parent / "native_lean" if lean else BUILD.parent / "native_checked" if checked else BUILD
     bdir.mkdir(parents=True, exist_ok=True)
     headers = _headers()
     common = ["-O3", "-fPIC", "-std=c++17", f"-I{CSRC}", f"-D_GLIBCXX_USE_CXX11_ABI={int(cxx11)}"]
     if checked:
         common += ["-DK8S_CHECKED", "-DK8S_MODULE_NAME=_C_checked"]
+    if lean:
+        common += ["-DK8S_LEAN", "-DK8S_MODULE_NAME=_C_lean"]
     py_inc = sysconfig.get_paths()["include"]
     units = []
     for src in sorted((CSRC / "kernels").glob("*.hip")):
+        if lean and src.name not in LEAN_KERNELS:
+            continue
         units.append((src, ["-x", "hip", f"--offload-arch={ARCH}", "-munsafe-fp-atomics",
                             *(NO_PACKED_FP32 if src.name in NO_PACKED_FP32_FILES else [])]))
     for src in sorted((CSRC / "runtime").glob("*.cpp")):
+        if lean and src.name not in LEAN_RUNTIME:
+            continue
         units.append((src, []))
     units.append((CSRC / "bindings.cpp", [f"-I{pybind11.get_include()}", f"-I{py_inc}", "-fvisibility=hidden"]))
     units.append((CSRC / "torch_stream.cpp", [f"-I{tinc}", f"-I{tinc / 'torch/csrc/api/include'}",
@@ -97,11 +113,12 @@ def build(jobs: int = 0, force: bool = False, verbose: bool = False, checked: bo
     with cf.ThreadPoolExecutor(max_workers=n) as ex:
         for f in [ex.submit(_run, c, verbose) for c in todo]:
             f.result()
-    out = ext_path(checked)
+    out = ext_path(checked, lean)
     if todo or force or not out.exists() or any(o.stat().st_mtime > out.stat().st_mtime for o in objs):
         tmp = out.with_suffix(".tmp.so")
         _run([HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", str(tmp), *map(str, objs),
-              f"-L{tlib}", "-lc10_hip", "-lc10", "-lrccl", f"-Wl,-rpath,{tlib}", "-Wl,--no-as-needed"], verbose)
+              f"-L{tlib}", "-lc10_hip", "-lc10", *([] if lean else ["-lrccl"]), f"-Wl,-rpath,{tlib}",
+              "-Wl,--no-as-needed"], verbose)
         os.replace(tmp, out)
     return out
 
@@ -112,8 +129,9 @@ def main(argv=None) -> int:
     ap.add_argument("--force", action="store_true")
     ap.add_argument("-v", "--verbose", action="store_true")
     ap.add_argument("--checked", action="store_true", help="bounds-checked kernels: ops/_C_checked*.so")
+    ap.add_argument("--lean", action="store_true", help="runtime + fp32-stream model kernels only: ops/_C_lean*.so")
     a = ap.parse_args(argv)
-    p = build(a.jobs, a.force, a.verbose, a.checked)
+    p = build(a.jobs, a.force, a.verbose, a.checked, a.lean)
     print(p)
     return 0
 

@@ -16,8 +16,10 @@
 #include <string>
 
 #include "runtime/block_allocator.h"
+#ifndef K8S_LEAN
 #include "runtime/rccl_comm.h"
 #include "runtime/xgmi_comm.h"
+#endif
 
 namespace py = pybind11;
 
@@ -211,16 +213,29 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
   // point every instrumented unit at one device record (ops.check_*); returns 0, or nonzero in release builds
   m.def("check_bind", [](uintptr_t rec) {
     int rc = 0;
+#ifdef K8S_LEAN
+    rc |= k8s_check_bind_misc(reinterpret_cast<void*>(rec));
+#else
     for (auto f : {k8s_check_bind_misc, k8s_check_bind_rope_kv, k8s_check_bind_attn_decode_fused,
                    k8s_check_bind_attn_decode_split, k8s_check_bind_attn_prefill, k8s_check_bind_attn_decode})
       rc |= f(reinterpret_cast<void*>(rec));
+#endif
     return rc;
   });
   m.doc() = "gfx950 HIP kernels and native runtime of k8s_llm_scheduler_amd";
   m.attr("ARCH") = "gfx950";
+  // The lean module (-DK8S_LEAN: python -m k8s_llm_scheduler_amd._build --lean) holds the runtime, the sampler and the
+  // kernels of the fp32-stream models only; the tuned GEMV / GEMM kernels, the Llama attention kernels, fp8 and the
+  // communicators are left out, and the any-shape GEMM serves every product.
+#ifdef K8S_LEAN
+  m.attr("lean") = true;
+#else
+  m.attr("lean") = false;
+#endif
 
   m.def("rmsnorm", [](uintptr_t out, uintptr_t x, uintptr_t residual, uintptr_t w, int rows, int H, float eps,
                       int64_t s) { check(k8s_rmsnorm(P(out), P(x), P(residual), P(w), rows, H, eps, S(s)), "rmsnorm"); });
+#ifndef K8S_LEAN
   m.def("rope_kv_write", [](uintptr_t q_out, uintptr_t kc, uintptr_t vc, uintptr_t qkv, uintptr_t cos_sin,
                             uintptr_t pos, uintptr_t slots, uintptr_t ctx, uintptr_t bt, int max_blocks, int bs, int T,
                             int nq, int nkv, int D, int64_t s) {
@@ -242,6 +257,7 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
                                       max_qlen, nq, nkv, D, bs, max_blocks, S(s)),
           "paged_prefill_attention");
   });
+#endif
   // Bounded wait for a recorded hipEvent (torch.cuda.Event.cuda_event) with the GIL released: the engine's per-step
   // device waits must neither block forever (a stalled collective) nor hold the GIL while they poll (the control
   // plane's watch / worker threads run beside the engine loop).  True once the event completed, False at the timeout.
@@ -259,6 +275,7 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
       else std::this_thread::sleep_for(std::chrono::microseconds(50));
     }
   }, py::arg("event"), py::arg("timeout_s"));
+#ifndef K8S_LEAN
   m.def("pgemm_set_prio", [](int mode) { return k8s_pgemm_set_prio(mode); });
   m.def("pgemm_set_row_slabs", [](int on) { return k8s_pgemm_set_row_slabs(on); });
   m.def("gemv_set_wide", [](int on) { return k8s_gemv_set_wide(on); });
@@ -343,6 +360,7 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
                                      P<int>(bt), P<int>(ctx), scale, B, nq, nkv, D, bs, max_blocks, pmax, S(s)),
           "decode_attention_split");
   });
+#endif
   m.def("sample", [](uintptr_t tokens, uintptr_t logits, int B, int Vs, int shards, uintptr_t temp, uintptr_t top_p,
                      uintptr_t seeds, uintptr_t counter, uintptr_t ctx_inc, uintptr_t hist, int hist_stride,
                      uintptr_t steps, uintptr_t scratch, uintptr_t nuc_scratch, uintptr_t slots, uintptr_t cls,
@@ -536,6 +554,7 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
                           f32, S(s)), "moe_combine");
   });
 
+#ifndef K8S_LEAN
   m.def("mgemm_configs", []() {
     py::list out;
     for (int c = 0; c < k8s_mgemm_num_configs(); ++c) {
@@ -680,6 +699,7 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
       .def_property("twoshot_min_bytes", &XgmiComm::twoshot_min_bytes, &XgmiComm::set_twoshot_min_bytes)
       .def_property_readonly("max_allreduce_bytes", &XgmiComm::max_allreduce_bytes);
 
+#endif
   using k8sllm::BlockAllocator;
   py::class_<BlockAllocator::Allocation>(m, "Allocation")
       .def_readonly("blocks", &BlockAllocator::Allocation::blocks)

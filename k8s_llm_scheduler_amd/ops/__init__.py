@@ -27,6 +27,15 @@ try:  # torch must be imported first: the extension binds to torch's HIP runtime
     _C = importlib.import_module("k8s_llm_scheduler_amd.ops._C_checked" if CHECKED else "k8s_llm_scheduler_amd.ops._C")
 except Exception as e:  # pragma: no cover - reported loudly on first GPU use
     _C_ERR = e
+    if not CHECKED:
+        # the lean module (python -m k8s_llm_scheduler_amd._build --lean): runtime, sampler and the kernels of the
+        # fp32-stream model designs; the Llama path and the tuned GEMMs need the full module
+        try:
+            _C = importlib.import_module("k8s_llm_scheduler_amd.ops._C_lean")
+        except Exception:  # noqa: BLE001 -- the full module's error is the one to report
+            pass
+# True when only the lean module is loaded: ops of the Llama path raise, seqmix keeps every product on its own GEMM
+LEAN = bool(getattr(_C, "lean", False))
 
 EPI_BF16, EPI_F32, EPI_SWIGLU = 0, 1, 2
 BF16, F32, I32 = torch.bfloat16, torch.float32, torch.int32

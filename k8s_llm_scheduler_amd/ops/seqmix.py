@@ -113,8 +113,10 @@ def _route_fast(a: torch.Tensor, w: torch.Tensor, out_dtype) -> bool:
     """bf16 products of production size whose shape the framework's tuned GEMV / MFMA GEMM kernels take (128-byte
     k steps, N % 16 == 0, at least 1024 x 512 weights: the sizes their plan tables and heuristics were tuned and
     tested on).  Smaller products are launch-bound and stay on the any-shape kernel."""
-    from . import GEMM_BACKEND
+    from . import GEMM_BACKEND, LEAN
 
+    if LEAN:
+        return False
     if a.dtype != BF16 or w.dtype != BF16 or out_dtype not in (BF16, F32) or a.dim() != 2 or w.dim() != 2:
         return False
     if GEMM_BACKEND == "library" or not a.is_contiguous() or not w.is_contiguous():
