@@ -23,19 +23,30 @@ _C_ERR: Optional[BaseException] = None
 # K8S_CHECKED=1 loads the bounds-checked build (python -m k8s_llm_scheduler_amd._build --checked): kernels range-check
 # every index they derive from data and record violations, which the engine raises after each step (check_raise)
 CHECKED = os.environ.get("K8S_CHECKED", "0") == "1"
-try:  # torch must be imported first: the extension binds to torch's HIP runtime
-    _C = importlib.import_module("k8s_llm_scheduler_amd.ops._C_checked" if CHECKED else "k8s_llm_scheduler_amd.ops._C")
-except Exception as e:  # pragma: no cover - reported loudly on first GPU use
-    _C_ERR = e
-    if not CHECKED:
-        # the lean module (python -m k8s_llm_scheduler_amd._build --lean): runtime, sampler and the kernels of the
-        # fp32-stream model designs; the Llama path and the tuned GEMMs need the full module
-        try:
-            _C = importlib.import_module("k8s_llm_scheduler_amd.ops._C_lean")
-        except Exception:  # noqa: BLE001 -- the full module's error is the one to report
-            pass
 # True when only the lean module is loaded: ops of the Llama path raise, seqmix keeps every product on its own GEMM
-LEAN = bool(getattr(_C, "lean", False))
+LEAN = False
+
+
+def _load() -> None:
+    """Import the extension: the full module, else (python -m k8s_llm_scheduler_amd._build --lean) the lean one with the
+    runtime, the sampler and the kernels of the fp32-stream model designs.  Called at import and again by native() /
+    available() while nothing is loaded, so a module built after this package was imported is picked up."""
+    global _C, _C_ERR, LEAN
+    try:  # torch must be imported first: the extension binds to torch's HIP runtime
+        _C = importlib.import_module("k8s_llm_scheduler_amd.ops._C_checked" if CHECKED
+                                     else "k8s_llm_scheduler_amd.ops._C")
+    except Exception as e:  # pragma: no cover - reported loudly on first GPU use
+        _C_ERR = e
+        if not CHECKED:
+            try:
+                importlib.invalidate_caches()
+                _C = importlib.import_module("k8s_llm_scheduler_amd.ops._C_lean")
+            except Exception:  # noqa: BLE001 -- the full module's error is the one to report
+                pass
+    LEAN = bool(getattr(_C, "lean", False))
+
+
+_load()
 
 EPI_BF16, EPI_F32, EPI_SWIGLU = 0, 1, 2
 BF16, F32, I32 = torch.bfloat16, torch.float32, torch.int32
@@ -57,12 +68,16 @@ def _split_pairs_limit(max_context: int) -> int:
 def native():
     """The loaded extension module; raises with the build hint if it is missing."""
     if _C is None:
+        _load()
+    if _C is None:
         raise RuntimeError("k8s_llm_scheduler_amd native extension (_C) is not built/loadable: "
                            f"{_C_ERR!r}. Run: python -m k8s_llm_scheduler_amd._build")
     return _C
 
 
 def available() -> bool:
+    if _C is None:
+        _load()
     return _C is not None
 
 
