@@ -327,7 +327,7 @@ __global__ void window_merge_kernel(TA* __restrict__ out, const float* __restric
 //   S^T[key][column] = K Q^T      A = 16 staged key rows, B = the columns' queries (registers)
 //   O[column][d]    += P V        A = the 32 keys' probabilities (registers, keys in the order the S^T tiles left
 //                                 them), B = the staged value columns through the transposing LDS read
-// scores, softmax and sums in fp32; a sink starts every column at (max 0, sum 1).
+// scores, softmax and sums in fp32, the weights applied as two bf16 terms; a sink starts every column at (max 0, sum 1).
 typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
 
 template <int NKK, int NVB, int NCB>
@@ -489,11 +489,14 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
       float a_i[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) a_i[i] = __shfl(alpha, g4 * 4 + i, WAVE);
-      bf16x8 pa;       // slot j < 4: key 4 g4 + j; slot j >= 4: key 16 + 4 g4 + (j - 4)
+      // the fp32 weights enter the product as two bf16 terms (p = hi + lo, |lo| <= 2^-9 p): 16 bits of each weight
+      bf16x8 pa, pl;   // slot j < 4: key 4 g4 + j; slot j >= 4: key 16 + 4 g4 + (j - 4)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         pa[j] = (__bf16)sacc[0][j];
         pa[4 + j] = (__bf16)sacc[1][j];
+        pl[j] = (__bf16)(sacc[0][j] - (float)pa[j]);
+        pl[4 + j] = (__bf16)(sacc[1][j] - (float)pa[4 + j]);
       }
       const int r0 = 4 * g4 + qd, r1 = r0 + 16;
 #pragma unroll
@@ -508,6 +511,7 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
 #pragma unroll
           for (int j = 0; j < 4; ++j) { vb[j] = v0[j]; vb[4 + j] = v1[j]; }
           o[cb][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vb, o[cb][n], 0, 0, 0);
+          o[cb][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pl, vb, o[cb][n], 0, 0, 0);
         }
       }
     }

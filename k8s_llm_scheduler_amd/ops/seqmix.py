@@ -432,13 +432,14 @@ WINDOW_MFMA = os.environ.get("K8S_WINDOW_MFMA", "1") != "0"   # 0: always the pl
 
 
 def window_splits(T: int, G: int, window: int, P: int, max_pos: int, tile_rows: int) -> int:
-    """Key splits of the plain windowed attention: one when the (token, key head) grid fills the chip by itself, else
-    enough splits of at least one tile each for about 256 workgroups.  ``max_pos``: positions a token can have."""
+    """Key splits of the plain windowed attention: one when the (token, key head) grid fills the chip several times over
+    by itself, else enough splits of at least one tile each for about 1024 workgroups (a workgroup walks its tiles one
+    after the other, so decoding wants them spread).  ``max_pos``: positions a token can have."""
     groups = T * G
-    if groups >= 128 or tile_rows <= 0:
+    if groups >= 1024 or tile_rows <= 0:
         return 1
     keys = max_pos if window <= 0 else min(max_pos, window + (max_pos // P if P > 0 else 0))
-    return max(1, min(256 // groups, -(-max(1, keys) // tile_rows), 16))
+    return max(1, min(-(-1024 // groups), -(-max(1, keys) // tile_rows), 16))
 
 
 def window_attention(q: torch.Tensor, gate: Optional[torch.Tensor], kcache: torch.Tensor, vcache: torch.Tensor,
