@@ -113,6 +113,7 @@ __global__ __launch_bounds__(256) void window_pool_kernel(float* __restrict__ kp
   const int GD = G * D, GV = G * V;
   for (int i = threadIdx.x; i < GD + GV; i += blockDim.x) {
     float a = 0.f;
+#pragma unroll 4
     for (int j = b * P; j < b * P + P; ++j) {
       const size_t slot = (size_t)btr[j / bs] * bs + (j % bs);
       a += i < GD ? ldf(kcache, slot * GD + i) : ldf(vcache, slot * GV + (i - GD));
@@ -435,23 +436,28 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
       if (u0 + 31 >= nb_max && j_first <= w_pmax && j_last >= w_lo) any = true;
     }
     if (!any) continue;
+    // every staged key fragment is read once and serves all column blocks of the wave
+    f32x4 sacc[NCB][2];
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+#pragma unroll
+      for (int cb = 0; cb < NCB; ++cb) sacc[cb][m] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < NKK; ++kk) {
+        if (kk < nkk) {
+          const int piece = 32 * kk + 8 * g4;
+          bf16x8 ka = __builtin_bit_cast(bf16x8, zero);
+          if (piece < D) ka = *reinterpret_cast<const bf16x8*>(klds + (16 * m + li) * rowk + 2 * piece);
+#pragma unroll
+          for (int cb = 0; cb < NCB; ++cb)
+            sacc[cb][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[cb][kk], sacc[cb][m], 0, 0, 0);
+        }
+      }
+    }   // sacc[cb][m][i] = S[key u0 + 16 m + 4 g4 + i][column li of block cb]
+    bf16x8 pa[NCB], pl[NCB];   // slot j < 4: key 4 g4 + j; slot j >= 4: key 16 + 4 g4 + (j - 4)
+    float a_i[NCB][4];
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) {
-      f32x4 sacc[2];
-#pragma unroll
-      for (int m = 0; m < 2; ++m) {
-        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int kk = 0; kk < NKK; ++kk) {
-          if (kk < nkk) {
-            const int piece = 32 * kk + 8 * g4;
-            bf16x8 ka = __builtin_bit_cast(bf16x8, zero);
-            if (piece < D) ka = *reinterpret_cast<const bf16x8*>(klds + (16 * m + li) * rowk + 2 * piece);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[cb][kk], acc, 0, 0, 0);
-          }
-        }
-        sacc[m] = acc;   // S[key u0 + 16 m + 4 g4 + i][column li]
-      }
       float tmax = -INFINITY;
 #pragma unroll
       for (int m = 0; m < 2; ++m)
@@ -464,8 +470,8 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
             const int j = lo_min + (u - nb_max);
             vis = j <= c_p[cb] && j >= c_lo[cb];
           }
-          const float v = vis ? sacc[m][i] * scale : -INFINITY;
-          sacc[m][i] = v;
+          const float v = vis ? sacc[cb][m][i] * scale : -INFINITY;
+          sacc[cb][m][i] = v;
           tmax = fmaxf(tmax, v);
         }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
@@ -478,40 +484,41 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
       for (int m = 0; m < 2; ++m)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float pv = expf(sacc[m][i] - m_ref);
-          sacc[m][i] = pv;
+          const float pv = expf(sacc[cb][m][i] - m_ref);
+          sacc[cb][m][i] = pv;
           rsum += pv;
         }
       rsum += __shfl_xor(rsum, 16, WAVE);
       rsum += __shfl_xor(rsum, 32, WAVE);
       l_run[cb] = l_run[cb] * alpha + rsum;
       m_run[cb] = m_new;
-      float a_i[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) a_i[i] = __shfl(alpha, g4 * 4 + i, WAVE);
+      for (int i = 0; i < 4; ++i) a_i[cb][i] = __shfl(alpha, g4 * 4 + i, WAVE);
       // the fp32 weights enter the product as two bf16 terms (p = hi + lo, |lo| <= 2^-9 p): 16 bits of each weight
-      bf16x8 pa, pl;   // slot j < 4: key 4 g4 + j; slot j >= 4: key 16 + 4 g4 + (j - 4)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        pa[j] = (__bf16)sacc[0][j];
-        pa[4 + j] = (__bf16)sacc[1][j];
-        pl[j] = (__bf16)(sacc[0][j] - (float)pa[j]);
-        pl[4 + j] = (__bf16)(sacc[1][j] - (float)pa[4 + j]);
+        pa[cb][j] = (__bf16)sacc[cb][0][j];
+        pa[cb][4 + j] = (__bf16)sacc[cb][1][j];
+        pl[cb][j] = (__bf16)(sacc[cb][0][j] - (float)pa[cb][j]);
+        pl[cb][4 + j] = (__bf16)(sacc[cb][1][j] - (float)pa[cb][4 + j]);
       }
-      const int r0 = 4 * g4 + qd, r1 = r0 + 16;
+    }
+    const int r0 = 4 * g4 + qd, r1 = r0 + 16;
 #pragma unroll
-      for (int n = 0; n < NVB; ++n) {
-        if (n < nvb) {
+    for (int n = 0; n < NVB; ++n) {
+      if (n < nvb) {
+        const int col = 16 * n + 4 * pd;
+        const bf16x4 v0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(vlds + r0 * rowv + 2 * col));
+        const bf16x4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(vlds + r1 * rowv + 2 * col));
+        bf16x8 vb;
 #pragma unroll
-          for (int i = 0; i < 4; ++i) o[cb][n][i] *= a_i[i];
-          const int col = 16 * n + 4 * pd;
-          const bf16x4 v0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(vlds + r0 * rowv + 2 * col));
-          const bf16x4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(vlds + r1 * rowv + 2 * col));
-          bf16x8 vb;
+        for (int j = 0; j < 4; ++j) { vb[j] = v0[j]; vb[4 + j] = v1[j]; }
 #pragma unroll
-          for (int j = 0; j < 4; ++j) { vb[j] = v0[j]; vb[4 + j] = v1[j]; }
-          o[cb][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vb, o[cb][n], 0, 0, 0);
-          o[cb][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pl, vb, o[cb][n], 0, 0, 0);
+        for (int cb = 0; cb < NCB; ++cb) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[cb][n][i] *= a_i[cb][i];
+          o[cb][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[cb], vb, o[cb][n], 0, 0, 0);
+          o[cb][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pl[cb], vb, o[cb][n], 0, 0, 0);
         }
       }
     }
