@@ -92,7 +92,7 @@ __device__ __forceinline__ size_t pool_entry(const int* btr, int b, int P, int b
   return (size_t)btr[page] * ppb + (b - first);
 }
 
-// One workgroup per token; works only for tokens that end a block of P ((pos + 1) % P == 0): the mean, in fp32, of the
+// Workgroups (token, slice of the row); only tokens that end a block of P work ((pos + 1) % P == 0): the mean, in fp32, of the
 // P cached keys and values (as the cache holds them) -> kpool / vpool [pages * ppb][G][D or V] fp32.  Runs after the
 // cache write of the same batch, so the block's earlier tokens are in the cache whether this batch or an earlier one
 // brought them.
@@ -111,7 +111,7 @@ __global__ __launch_bounds__(256) void window_pool_kernel(float* __restrict__ kp
   const size_t e = pool_entry(btr, b, P, bs, ppb);
   const float invp = 1.0f / (float)P;
   const int GD = G * D, GV = G * V;
-  for (int i = threadIdx.x; i < GD + GV; i += blockDim.x) {
+  for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < GD + GV; i += gridDim.y * blockDim.x) {
     float a = 0.f;
 #pragma unroll 4
     for (int j = b * P; j < b * P + P; ++j) {
@@ -576,12 +576,14 @@ extern "C" int k8s_window_pool(float* kpool, float* vpool, const void* kcache, c
   if (T <= 0 || P <= 0) return 0;
   if (G <= 0 || D <= 0 || V <= 0 || bs <= 0) return -1;
   const int ppb = (bs + P - 1) / P;
+  const int slices = (G * (D + V) + 255) / 256;
+  const dim3 grid(T, slices < 16 ? slices : 16);
   if (f32)
-    window_pool_kernel<float><<<T, 256, 0, s>>>(kpool, vpool, (const float*)kcache, (const float*)vcache, block_tables,
-                                                max_blocks, tok_seq, positions, G, D, V, P, bs, ppb);
+    window_pool_kernel<float><<<grid, 256, 0, s>>>(kpool, vpool, (const float*)kcache, (const float*)vcache,
+                                                   block_tables, max_blocks, tok_seq, positions, G, D, V, P, bs, ppb);
   else
-    window_pool_kernel<bf16_t><<<T, 256, 0, s>>>(kpool, vpool, (const bf16_t*)kcache, (const bf16_t*)vcache,
-                                                 block_tables, max_blocks, tok_seq, positions, G, D, V, P, bs, ppb);
+    window_pool_kernel<bf16_t><<<grid, 256, 0, s>>>(kpool, vpool, (const bf16_t*)kcache, (const bf16_t*)vcache,
+                                                    block_tables, max_blocks, tok_seq, positions, G, D, V, P, bs, ppb);
   return (int)hipGetLastError();
 }
 
