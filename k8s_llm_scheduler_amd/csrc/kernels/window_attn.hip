@@ -331,7 +331,7 @@ __global__ void window_merge_kernel(TA* __restrict__ out, const float* __restric
 // scores, softmax and sums in fp32, the weights applied as two bf16 terms; a sink starts every column at (max 0, sum 1).
 typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
 
-template <int NKK, int NVB, int NCB>
+template <int NKK, int NVB, int NCB, bool PF>
 __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long ldq, const bf16_t* __restrict__ gate, long ldg,
     const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache, const float* __restrict__ kpool,
@@ -406,28 +406,76 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
     for (int n = 0; n < NVB; ++n) o[cb][n] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   const int qd = li >> 2, pd = li & 3;
+  // Staging: every thread moves NST 16-byte chunks of a step's 32 rows.  PF: the chunks of step s + 1 are loaded into
+  // registers before step s is computed and written to LDS after it, so the cache reads run under the MFMAs -- for
+  // grids of at most one workgroup per CU, where nothing else hides them; larger grids run the variant without the
+  // held registers, at twice the waves per SIMD.
+  constexpr int NST = (NKK * 4 + NVB * 2 + 7) / 8;
+  u32x4 pre[NST];
+  auto stage_load = [&](int u0) {
+#pragma unroll
+    for (int i = 0; i < NST; ++i) {
+      const int idx = tid + 256 * i;
+      u32x4 v = zero;
+      if (idx < 32 * cpr) {
+        const int r = idx / cpr, c = idx - r * cpr, u = u0 + r;
+        const bool isk = c < ckd;
+        const int e8 = 8 * (isk ? c : c - ckd);
+        if (u < nb_max) {
+          const size_t e = pool_entry(btr, u, P, bs, ppb);
+          const float* src = isk ? kpool + e * GD + (size_t)g * D + e8 : vpool + e * GV + (size_t)g * V + e8;
+          const f32x4 a = *reinterpret_cast<const f32x4*>(src), b = *reinterpret_cast<const f32x4*>(src + 4);
+          v = u32x4{pack_bf2(a[0], a[1]), pack_bf2(a[2], a[3]), pack_bf2(b[0], b[1]), pack_bf2(b[2], b[3])};
+        } else if (u < nkeys) {
+          const int j = lo_min + (u - nb_max);
+          const size_t slot = (size_t)btr[j / bs] * bs + (j % bs);
+          v = isk ? *reinterpret_cast<const u32x4*>(kcache + slot * GD + (size_t)g * D + e8)
+                  : *reinterpret_cast<const u32x4*>(vcache + slot * GV + (size_t)g * V + e8);
+        }
+      }
+      pre[i] = v;
+    }
+  };
+  auto stage_store = [&]() {
+#pragma unroll
+    for (int i = 0; i < NST; ++i) {
+      const int idx = tid + 256 * i;
+      if (idx < 32 * cpr) {
+        const int r = idx / cpr, c = idx - r * cpr;
+        const bool isk = c < ckd;
+        const int e8 = 8 * (isk ? c : c - ckd);
+        *reinterpret_cast<u32x4*>((isk ? klds + r * rowk : vlds + r * rowv) + 2 * e8) = pre[i];
+      }
+    }
+  };
+  if (PF) stage_load(0);
   for (int step = 0; step < nsteps; ++step) {
     const int u0 = step * 32;
-    __syncthreads();
-    for (int idx = tid; idx < 32 * cpr; idx += 256) {
-      const int r = idx / cpr, c = idx - r * cpr, u = u0 + r;
-      const bool isk = c < ckd;
-      const int e8 = 8 * (isk ? c : c - ckd);
-      u32x4 v = zero;
-      if (u < nb_max) {
-        const size_t e = pool_entry(btr, u, P, bs, ppb);
-        const float* src = isk ? kpool + e * GD + (size_t)g * D + e8 : vpool + e * GV + (size_t)g * V + e8;
-        const f32x4 a = *reinterpret_cast<const f32x4*>(src), b = *reinterpret_cast<const f32x4*>(src + 4);
-        v = u32x4{pack_bf2(a[0], a[1]), pack_bf2(a[2], a[3]), pack_bf2(b[0], b[1]), pack_bf2(b[2], b[3])};
-      } else if (u < nkeys) {
-        const int j = lo_min + (u - nb_max);
-        const size_t slot = (size_t)btr[j / bs] * bs + (j % bs);
-        v = isk ? *reinterpret_cast<const u32x4*>(kcache + slot * GD + (size_t)g * D + e8)
-                : *reinterpret_cast<const u32x4*>(vcache + slot * GV + (size_t)g * V + e8);
+    __syncthreads();          // the previous step's fragments have been read
+    if (PF) {
+      stage_store();
+    } else {                  // chunk by chunk: no registers held across the step
+      for (int idx = tid; idx < 32 * cpr; idx += 256) {
+        const int r = idx / cpr, c = idx - r * cpr, u = u0 + r;
+        const bool isk = c < ckd;
+        const int e8 = 8 * (isk ? c : c - ckd);
+        u32x4 v = zero;
+        if (u < nb_max) {
+          const size_t e = pool_entry(btr, u, P, bs, ppb);
+          const float* src = isk ? kpool + e * GD + (size_t)g * D + e8 : vpool + e * GV + (size_t)g * V + e8;
+          const f32x4 a = *reinterpret_cast<const f32x4*>(src), b = *reinterpret_cast<const f32x4*>(src + 4);
+          v = u32x4{pack_bf2(a[0], a[1]), pack_bf2(a[2], a[3]), pack_bf2(b[0], b[1]), pack_bf2(b[2], b[3])};
+        } else if (u < nkeys) {
+          const int j = lo_min + (u - nb_max);
+          const size_t slot = (size_t)btr[j / bs] * bs + (j % bs);
+          v = isk ? *reinterpret_cast<const u32x4*>(kcache + slot * GD + (size_t)g * D + e8)
+                  : *reinterpret_cast<const u32x4*>(vcache + slot * GV + (size_t)g * V + e8);
+        }
+        *reinterpret_cast<u32x4*>((isk ? klds + r * rowk : vlds + r * rowv) + 2 * e8) = v;
       }
-      *reinterpret_cast<u32x4*>((isk ? klds + r * rowk : vlds + r * rowv) + 2 * e8) = v;
     }
     __syncthreads();
+    if (PF && step + 1 < nsteps) stage_load(u0 + 32);
     // keys of this step that any column of the wave can see: pooled blocks below w_nb, tokens w_lo .. w_pmax
     bool any = false;
     if (w_any) {
@@ -666,13 +714,27 @@ extern "C" int k8s_window_attention_mfma(void* out, const void* q, long ldq, con
   constexpr int NCB = 2;
   const int TPB = 4 * NCB * (16 / R);
   const dim3 grid((max_qlen + TPB - 1) / TPB, G, nseq);
-#define K8S_WM(NKK, NVB)                                                                                              \
-  window_attention_mfma_kernel<NKK, NVB, NCB><<<grid, 256, lds, s>>>(                                                 \
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cus = n;
+  }
+  const bool pf = (long)grid.x * grid.y * grid.z <= cus;
+#define K8S_WM_P(NKK, NVB, PF)                                                                                        \
+  window_attention_mfma_kernel<NKK, NVB, NCB, PF><<<grid, 256, lds, s>>>(                                             \
       (bf16_t*)out, (const bf16_t*)q, ldq, (const bf16_t*)gate, ldg, (const bf16_t*)kcache, (const bf16_t*)vcache,    \
       kpool, vpool, block_tables, max_blocks, cu_q, positions, H, G, D, V, window, P, scale, sink, bs, ppb, R)
+#define K8S_WM(NKK, NVB)               \
+  do {                                 \
+    if (pf) K8S_WM_P(NKK, NVB, true);  \
+    else K8S_WM_P(NKK, NVB, false);    \
+  } while (0)
   if (D <= 64 && V <= 64) K8S_WM(2, 4);
   else if (D <= 128 && V <= 128) K8S_WM(4, 8);
-  else K8S_WM(8, 16);
+  else K8S_WM_P(8, 16, false);
 #undef K8S_WM
+#undef K8S_WM_P
   return (int)hipGetLastError();
 }
