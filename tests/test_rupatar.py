@@ -399,7 +399,7 @@ OTHER_SIZES = [
             hgrn2(heads=1, dim=4, vdim=1), mlstm(heads=1, dim=2, vdim=1, cap=1.0)], width=8, vocab=11, groups=8),
     # aligned sizes with mixers of different widths in one model
     config([with_mlp(attn(heads=8, kv_heads=4, dim=32, vdim=16, window=33, pool=16, dims=32, scale=0.18), moe(experts=4, top=2, ff=32, shared=64)),
-            hgrn2(heads=4, dim=16, vdim=32), mlstm(heads=2, dim=64, vdim=64, cap=12.0),
+            hgrn2(heads=4, dim=16, vdim=32), mlstm(heads=2, dim=64, vdim=64, cap=11.0),
             with_mlp(attn(heads=8, kv_heads=4, dim=64, vdim=16, window=64, pool=32, dims=16, scale=0.125), moe(experts=8, top=8, ff=16, shared=0))],
            width=64, vocab=80, groups=4),
 ]

@@ -315,7 +315,7 @@ def window_case(H, G, D, V, window, P, dims, dt, bs=16, seed=0):
 @pytest.mark.parametrize("H,G,D,V,window,P,dims", [
     (4, 2, 24, 20, 33, 5, 8),        # odd sizes: the plain kernel in both types
     (6, 2, 16, 16, 20, 16, 16),      # three query heads per key head: no matrix-core tiling
-    (8, 2, 64, 64, 40, 12, 32),      # matrix cores in bf16: four query heads per key head
+    (12, 3, 64, 64, 40, 10, 24),     # matrix cores in bf16: four query heads per key head
     (4, 4, 128, 128, 64, 7, 64),     # one query head per key head, 128-wide heads
     (16, 1, 32, 48, 17, 3, 0),       # sixteen query heads on one key head, no rotation
     (8, 4, 72, 80, 0, 0, 8),         # no window
@@ -331,11 +331,11 @@ def test_window_attention_ops(dt, tol, H, G, D, V, window, P, dims):
 
 def test_window_attention_matrix_cores_match_plain_kernel():
     """The same caches through both kernels in bf16 (the plain one is also the fp32 path)."""
-    outs, _ = window_case(8, 2, 64, 64, 40, 12, 32, torch.bfloat16, seed=3)
+    outs, _ = window_case(12, 3, 64, 64, 40, 10, 24, torch.bfloat16, seed=3)
     old = sm.WINDOW_MFMA
     try:
         sm.WINDOW_MFMA = False
-        plain, _ = window_case(8, 2, 64, 64, 40, 12, 32, torch.bfloat16, seed=3)
+        plain, _ = window_case(12, 3, 64, 64, 40, 10, 24, torch.bfloat16, seed=3)
     finally:
         sm.WINDOW_MFMA = old
     close(outs[DEV][1], plain[DEV][1], 2e-2)
