@@ -21,7 +21,8 @@ struct ScanCols { int q, k, v, i, f, g; };   // column offsets of the parts insi
 // [c CH, (c + 1) CH) of S; group c = 0 prepares each token's per-channel read / keep / write coefficients in LDS (and,
 // KIND 1, owns n).  The partial outputs of the channel groups meet in LDS; group 0 normalises and stores.  The next
 // token's inputs are loaded while the current one is computed; the barriers wait for LDS traffic only.
-// blockDim = (DX, NS): DX = max(D, V) rounded up to 64, NS = ceil(D / CH).  State record: S [D][V] (, n [D], m).
+// blockDim = (DX, NS): DX = max(D, V) rounded up to 64, NS = ceil(D / CH), CH (16, 32 or 64) the smallest that keeps
+// DX NS within 1024 threads.  State record: S [D][V] (, n [D], m).
 //
 // MODE 0: a whole portion per workgroup, from the slot's state (zero at position 0) to the slot's state.
 // Long portions run as three passes over chunks of Lc tokens, so the recurrence is parallel over chunks; a chunk record
@@ -44,10 +45,10 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
                                                           float eps, float cap, int nseq, int Lc,
                                                           float* __restrict__ cs_loc,
                                                           const float* __restrict__ cs_start) {
-  constexpr int DMAX = 128;
+  constexpr int DMAX = 256;
   __shared__ __attribute__((aligned(16))) float sq[DMAX], sa[DMAX], sb[DMAX];
   __shared__ float po[DMAX / CH][DMAX];
-  __shared__ float red[2], rednq[2];
+  __shared__ float red[4], rednq[4];
   const int hd = blockIdx.y;
   int s, a0, b0, p0;
   bool from_zero, last = true;
@@ -185,15 +186,17 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
       if (onv)
         for (int g = 0; g < NS; ++g) o += po[g][x];
       if (KIND == 1) {
-        const float nqs = rednq[0] + (D > 64 ? rednq[1] : 0.f);
+        float nqs = rednq[0];
+        for (int w = 1; w < (D + 63) / 64; ++w) nqs += rednq[w];
         o /= fmaxf(fabsf(nqs), expf(-m)) + 1e-6f;
       }
       ss = wave_sum(onv ? o * o : 0.f);
       if (DX > 64 && (x & 63) == 0) red[x >> 6] = ss;
     }
-    if (DX > 64) {                     // the channels span two waves: one more exchange (uniform branch)
+    if (DX > 64) {                     // the channels span several waves: one more exchange (uniform branch)
       lds_barrier();
-      ss = red[0] + red[1];
+      ss = red[0];
+      for (int w = 1; w < DX / 64; ++w) ss += red[w];
     }
     if (c == 0 && onv) {
       float y = o / sqrtf(ss / (float)V + eps) * nwx;
@@ -274,7 +277,7 @@ __global__ void gated_prefix_kernel(float* __restrict__ cs_start, const float* _
 
 using namespace k8sllm;
 
-extern "C" int k8s_gated_scan_max_dim() { return 128; }
+extern "C" int k8s_gated_scan_max_dim() { return 256; }
 
 // floats of one (slot, head) state record
 extern "C" long long k8s_gated_scan_record(int kind, int D, int V) {
@@ -294,21 +297,29 @@ extern "C" int k8s_gated_scan(void* out, const float* proj, long ld, int kind, i
                               float* state, const int* cu_q, const int* seq_slots, const int* positions, int nseq, int H,
                               int D, int V, float eps, float cap, int f32, int T, int Lc, float* ws, hipStream_t s) {
   if (nseq <= 0) return 0;
-  if (H <= 0 || H > 65535 || D <= 0 || D > 128 || V <= 0 || V > 128 || kind < 0 || kind > 1) return -1;
+  if (H <= 0 || H > 65535 || D <= 0 || D > 256 || V <= 0 || V > 256 || kind < 0 || kind > 1) return -1;
   if (kind == 0 && lower == nullptr) return -1;
   if (kind == 1 && !(cap > 0.f)) return -1;
-  constexpr int CH = 16;
-  const int m = D > V ? D : V;
-  const dim3 block((m + 63) / 64 * 64, (D + CH - 1) / CH);
+  const int m = D > V ? D : V, DX = (m + 63) / 64 * 64;
+  int ch = 16;
+  while (ch < 64 && DX * ((D + ch - 1) / ch) > 1024) ch *= 2;
+  if (DX * ((D + ch - 1) / ch) > 1024) return -2;
+  const dim3 block(DX, (D + ch - 1) / ch);
   const ScanCols co{cq, ck, cv, ci, cf, cg};
-#define K8S_GS(TA, KIND, MODE, GX, LOC, START)                                                                      \
+#define K8S_GS(TA, CH, KIND, MODE, GX, LOC, START)                                                                  \
   gated_scan_kernel<TA, CH, KIND, MODE><<<dim3(GX, H), block, 0, s>>>(                                              \
       (TA*)out, proj, ld, co, (const TA*)fbias, (const TA*)ibias, (const TA*)lower, (const TA*)normw, state, cu_q,  \
       seq_slots, positions, H, D, V, eps, cap, nseq, Lc, LOC, START)
+#define K8S_GS_C(TA, KIND, MODE, GX, LOC, START)                     \
+  do {                                                               \
+    if (ch == 16) K8S_GS(TA, 16, KIND, MODE, GX, LOC, START);        \
+    else if (ch == 32) K8S_GS(TA, 32, KIND, MODE, GX, LOC, START);   \
+    else K8S_GS(TA, 64, KIND, MODE, GX, LOC, START);                 \
+  } while (0)
 #define K8S_GS_K(TA, MODE, GX, LOC, START)                  \
   do {                                                      \
-    if (kind == 0) K8S_GS(TA, 0, MODE, GX, LOC, START);     \
-    else K8S_GS(TA, 1, MODE, GX, LOC, START);               \
+    if (kind == 0) K8S_GS_C(TA, 0, MODE, GX, LOC, START);   \
+    else K8S_GS_C(TA, 1, MODE, GX, LOC, START);             \
   } while (0)
 #define K8S_GS_T(MODE, GX, LOC, START)                      \
   do {                                                      \
@@ -330,6 +341,7 @@ extern "C" int k8s_gated_scan(void* out, const float* proj, long ld, int kind, i
   K8S_GS_T(2, chunks, nullptr, start);
 #undef K8S_GS_T
 #undef K8S_GS_K
+#undef K8S_GS_C
 #undef K8S_GS
   return (int)hipGetLastError();
 }

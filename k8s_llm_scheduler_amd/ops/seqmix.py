@@ -495,7 +495,7 @@ def window_attention(q: torch.Tensor, gate: Optional[torch.Tensor], kcache: torc
 
 # ----------------------------------------------------------------------------- gated matrix-state recurrences
 def gated_scan_max_dim() -> int:
-    return 128
+    return 256
 
 
 def gated_scan_record(kind: int, D: int, V: int) -> int:

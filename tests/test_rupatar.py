@@ -397,6 +397,9 @@ OTHER_SIZES = [
     # one of everything: one head, one expert, value size one, a pool longer than the window
     config([with_mlp(attn(heads=1, kv_heads=1, dim=4, vdim=1, window=3, pool=8, dims=4, scale=1.0), moe(experts=1, top=1, ff=4, shared=1)),
             hgrn2(heads=1, dim=4, vdim=1), mlstm(heads=1, dim=2, vdim=1, cap=1.0)], width=8, vocab=11, groups=8),
+    # recurrent heads wider than two waves: key channels in groups of 32 and 64
+    config([hgrn2(heads=1, dim=40, vdim=200), with_mlp(mlstm(heads=1, dim=144, vdim=136, cap=20.0), moe(experts=3, top=2, ff=8, shared=0)),
+            hgrn2(heads=2, dim=250, vdim=24)], width=48, vocab=31, groups=2),
     # aligned sizes with mixers of different widths in one model
     config([with_mlp(attn(heads=8, kv_heads=4, dim=32, vdim=16, window=33, pool=16, dims=32, scale=0.18), moe(experts=4, top=2, ff=32, shared=64)),
             hgrn2(heads=4, dim=16, vdim=32), mlstm(heads=2, dim=64, vdim=64, cap=11.0),

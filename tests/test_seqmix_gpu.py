@@ -344,7 +344,9 @@ def test_window_attention_matrix_cores_match_plain_kernel():
 # ----------------------------------------------------------------------------- gated matrix-state recurrences
 @pytest.mark.parametrize("dt,tol", DTYPES)
 @pytest.mark.parametrize("kind,H,D,V", [(sm.SCAN_HGRN2, 3, 20, 28), (sm.SCAN_HGRN2, 2, 64, 128), (sm.SCAN_HGRN2, 1, 100, 5),
-                                        (sm.SCAN_MLSTM, 3, 20, 28), (sm.SCAN_MLSTM, 2, 128, 64), (sm.SCAN_MLSTM, 5, 7, 70)])
+                                        (sm.SCAN_MLSTM, 3, 20, 28), (sm.SCAN_MLSTM, 2, 128, 64), (sm.SCAN_MLSTM, 5, 7, 70),
+                                        (sm.SCAN_HGRN2, 2, 128, 256), (sm.SCAN_MLSTM, 1, 256, 64), (sm.SCAN_MLSTM, 2, 160, 192),
+                                        (sm.SCAN_HGRN2, 1, 200, 136)])
 def test_gated_scan(dt, tol, kind, H, D, V):
     torch.manual_seed(30)
     cu, pos, slots, _ = batch()
